@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME,...] [--no-cpu]
+
+A "step" is one launch of the headline kernel -- the f16 4096^3 GEMM, the
+workload the reference's published numbers and BASELINE's MFMA target are quoted
+on -- over synthetic seeded inputs already resident in HBM.  K steps are timed
+between two stream synchronisations; the same region is also timed with HIP
+events on the launch stream (the events gpuLaunchKernel returns).  Every other
+BASELINE config is measured too and reported under "per_config", each with its
+own roofline fraction and single-core CPU baseline.
+
+Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, REPO)
+import __graft_entry__ as entry  # noqa: E402
+
+METRIC = "GEMM TFLOP/s (% MFMA peak) + softmax/reduce/transpose GB/s (% HBM peak), 1 GPU"
+HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X published dense f16 / bf16 MFMA rate
+FLUSH_BYTES = 512 << 20     # > L2 (8 x 4 MiB) + 256 MiB Infinity Cache
+
+
+def log(msg):
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
+class Workload:
+    """One BASELINE config: device buffers, the kernel launch, its algorithmic
+    work and the matching CPU-baseline call."""
+
+    def __init__(self, name, kernel, dims, bound, work, unit, dtype, describe):
+        self.name, self.kernel, self.dims = name, kernel, dims
+        self.bound, self.work, self.unit, self.dtype, self.describe = bound, work, unit, dtype, describe
+        self.args = None
+        self.buffers = []
+        self.cpu = None  # callable -> (value, sample description)
+
+
+def build_workloads(host, orc, stream, only):
+    wl = []
+
+    def want(name):
+        return only is None or name in only
+
+    def dev(a):
+        p = stream.to_device(a)
+        cur.buffers.append(p)
+        return p
+
+    def out(nbytes):
+        p = stream.alloc(nbytes)
+        cur.buffers.append(p)
+        return p
+
+    if want("gemm_f16_4096"):
+        M = N = K = 4096
+        cur = Workload("gemm_f16_4096", "imex_gemm_f16_f16_f32", [M, N, K], "mfma", 2.0 * M * N * K, "TFLOP/s",
+                       "f16", "C[4096,4096] f32 = A[4096,4096] f16 . B[4096,4096] f16, uniform(-1,1), seeds 20246/20247")
+        a = orc.fill_uniform(M * K, "f16", 20246, -1.0, 1.0).reshape(M, K)
+        b = orc.fill_uniform(K * N, "f16", 20247, -1.0, 1.0).reshape(K, N)
+        cur.args = [dev(a), dev(b), out(M * N * 4), M, N, K]
+        rows = 256
+
+        def cpu(a=a, b=b, rows=rows):
+            ms = orc.time_gemm_rows(a, b, rows, "f16")
+            return 2.0 * rows * N * K / (ms * 1e9), "first %d of 4096 rows of C, one un-warmed call of the i-k-j loop" % rows
+        cur.cpu = cpu
+        wl.append(cur)
+
+    if want("gemm_mlp_bf16"):
+        M, K, N = 4096, 4096, 11008
+        cur = Workload("gemm_mlp_bf16", "imex_gemm_bf16_bias_silu_bf16", [M, N, K], "mfma", 2.0 * M * N * K, "TFLOP/s",
+                       "bf16", "out[4096,11008] bf16 = silu(A[4096,4096] bf16 . B[4096,11008] bf16 + bias f32), seeds 20248-20250")
+        a = orc.fill_normal(M * K, "bf16", 20248, 0.0, 1.0).reshape(M, K)
+        b = orc.fill_normal(K * N, "bf16", 20249, 0.0, 0.02).reshape(K, N)
+        bias = orc.fill_normal(N, "f32", 20250, 0.0, 0.1)
+        cur.args = [dev(a), dev(b), dev(bias), out(M * N * 2), M, N, K]
+        rows = 64
+
+        def cpu(a=a, b=b, rows=rows):
+            ms = orc.time_gemm_rows(a, b, rows, "bf16")
+            return 2.0 * rows * N * K / (ms * 1e9), "first %d of 4096 rows, GEMM loop only" % rows
+        cur.cpu = cpu
+        wl.append(cur)
+
+    if want("relu_f32"):
+        n = 4096 * 4096
+        cur = Workload("relu_f32", "imex_relu_f32", [n], "hbm", 2.0 * n * 4, "GB/s", "f32",
+                       "relu f32 [4096,4096] uniform(-1,1) seed 20241, out of place")
+        x = orc.fill_uniform(n, "f32", 20241, -1.0, 1.0)
+        cur.args = [dev(x), out(n * 4), n]
+        cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_relu_f32(x, 2, 10) * 1e6), "full tensor, 2 warm-ups + 10 timed calls")
+        wl.append(cur)
+
+    if want("softmax_f16"):
+        rows, cols = 16384, 1024
+        cur = Workload("softmax_f16", "imex_softmax_f16", [rows, cols], "hbm", 2.0 * rows * cols * 2, "GB/s", "f16",
+                       "softmax f16 [16384,1024] normal(0,2) seed 20242, f32 internals")
+        x = orc.fill_normal(rows * cols, "f16", 20242, 0.0, 2.0).reshape(rows, cols)
+        cur.args = [dev(x), out(rows * cols * 2), rows, cols]
+        cur.cpu = lambda x=x: (2.0 * x.size * 2 / (orc.time_softmax_f16(x, 1, 3) * 1e6), "full tensor, 1 warm-up + 3 timed calls")
+        wl.append(cur)
+
+    if want("rowsum_f32"):
+        rows = cols = 8192
+        cur = Workload("rowsum_f32", "imex_rowsum_f32", [rows, cols], "hbm", rows * cols * 4.0 + rows * 4.0, "GB/s",
+                       "f32", "row-sum f32 [8192,8192] uniform(0,1) seed 20243 -> [8192]")
+        x = orc.fill_uniform(rows * cols, "f32", 20243, 0.0, 1.0).reshape(rows, cols)
+        cur.args = [dev(x), out(rows * 4), rows, cols, 0.0]
+        cur.cpu = lambda x=x: ((x.size * 4.0 + x.shape[0] * 4.0) / (orc.time_rowsum_f32(x, 1, 5) * 1e6), "full tensor, 1 warm-up + 5 timed calls")
+        wl.append(cur)
+
+    if want("transpose_bf16"):
+        rows = cols = 8192
+        cur = Workload("transpose_bf16", "imex_transpose2d_b16", [rows, cols], "hbm", 2.0 * rows * cols * 2, "GB/s",
+                       "bf16", "transpose bf16 [8192,8192] random non-NaN bits seed 20244")
+        x = orc.fill_bits(rows * cols, "bf16", 20244).reshape(rows, cols)
+        cur.args = [dev(x), out(rows * cols * 2), rows, cols]
+        cur.cpu = lambda x=x: (2.0 * x.size * 2 / (orc.time_transpose2d(x, 1, 3) * 1e6), "full tensor, 1 warm-up + 3 timed calls")
+        wl.append(cur)
+
+    if want("transpose_f32"):
+        rows = cols = 4096
+        cur = Workload("transpose_f32", "imex_transpose2d_b32", [rows, cols], "hbm", 2.0 * rows * cols * 4, "GB/s",
+                       "f32", "transpose f32 [4096,4096] random non-NaN bits seed 20245")
+        x = orc.fill_bits(rows * cols, "f32", 20245).reshape(rows, cols)
+        cur.args = [dev(x), out(rows * cols * 4), rows, cols]
+        cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_transpose2d(x, 1, 5) * 1e6), "full tensor, 1 warm-up + 5 timed calls")
+        wl.append(cur)
+
+    if want("silu_f32"):
+        n = 512 * 640 * 20 * 15
+        cur = Workload("silu_f32", "imex_silu_f32", [n], "hbm", 2.0 * n * 4, "GB/s", "f32",
+                       "silu f32 512x640x20x15 uniform(-8,8) seed 20251")
+        x = orc.fill_uniform(n, "f32", 20251, -8.0, 8.0)
+        cur.args = [dev(x), out(n * 4), n]
+        cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_silu_f32(x, 0, 2) * 1e6), "full tensor, 2 timed calls")
+        wl.append(cur)
+    return wl
+
+
+def roofline(w, ms):
+    if w.bound == "mfma":
+        achieved, peak, unit = w.work / (ms * 1e9), MFMA_PEAK_TFLOPS, "TFLOP/s"
+    else:
+        achieved, peak, unit = w.work / (ms * 1e6), HBM_PEAK_GBS, "GB/s"
+    return {"bound": w.bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": None}
+
+
+def measure_secondary(stream, w, rounds):
+    """Back-to-back launches (one event pair around all of them) and the
+    IMEX-profiler protocol with a cache flush before each timed launch."""
+    hot_total = stream.profile(w.kernel, w.dims, w.args, warmups=3, rounds=rounds, mode=1)[0]
+    hot_ms = hot_total / rounds
+    cold = stream.profile(w.kernel, w.dims, w.args, warmups=2, rounds=min(rounds, 20), flush_bytes=FLUSH_BYTES, mode=0)
+    cold_ms = float(np.median(cold))
+    return hot_ms, cold_ms
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--only", type=str, default=None, help="comma-separated workload names")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every kernel here runs on a single MI355X and this build has no "
+              "multi-GPU path (--gpus %d refused)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    only = set(args.only.split(",")) if args.only else None
+    if only is not None:
+        only.add("gemm_f16_4096")
+
+    pkg = entry.load_package()
+    host = pkg.host
+    orc = entry.load_oracle()
+    host.runtime()
+    host.kernels()  # raises if the HIP libraries are not built: there is no fallback
+
+    t_setup = time.time()
+    stream = host.Stream()
+    info = stream.device_info()
+    log("device: %s, %d CUs @ %.0f MHz" % (info["name"], info["cus"], info["clock_khz"] / 1e3))
+    workloads = build_workloads(host, orc, stream, only)
+    log("inputs generated and resident in HBM after %.1f s" % (time.time() - t_setup))
+
+    head = workloads[0]
+    K, W = args.steps, args.warmup
+    ev0 = None
+    for _ in range(max(W, 1)):
+        ev0 = stream.launch(head.kernel, head.dims, head.args)
+    stream.wait()
+    t0 = time.perf_counter()
+    ev1 = None
+    for _ in range(K):
+        ev1 = stream.launch(head.kernel, head.dims, head.args)
+    stream.wait()
+    t1 = time.perf_counter()
+    wall_ms = (t1 - t0) * 1e3 / K
+    # ev0 was recorded before the timed launches were enqueued (and the stream
+    # was idle at t0), so ev0 -> ev1 spans exactly the K timed launches.
+    event_ms = stream.elapsed_ms(ev0, ev1) / K
+    # device-side duration of a launch: back-to-back launches from C, no Python in the loop
+    kernel_ms = stream.profile(head.kernel, head.dims, head.args, warmups=3, rounds=K, mode=1)[0] / K
+    log("%s: wall %.4f ms/step, events %.4f ms/step, back-to-back %.4f ms/launch" % (head.name, wall_ms, event_ms, kernel_ms))
+    value = head.work / (wall_ms * 1e9)
+
+    result = {
+        "metric": METRIC, "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic (seeded std::mt19937 stream, inputs resident in HBM)",
+        "config": {"workload": "BASELINE configs[3]: " + head.describe, "kernel": head.kernel,
+                   "launch": "grid (256,1,1) x block (256,1,1)", "device": info["name"],
+                   "cus": info["cus"], "clock_mhz": info["clock_khz"] / 1e3},
+        "roofline": dict(roofline(head, kernel_ms), event_ms_per_step=round(event_ms, 5),
+                         kernel_ms=round(kernel_ms, 5)),
+    }
+
+    if not args.no_cpu and head.cpu:
+        t = time.time()
+        v, sample = head.cpu()
+        result["cpu_baseline"] = {"value": round(v, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                                  "sample": sample, "host_cores": os.cpu_count()}
+        log("cpu baseline %s: %.4f GFLOP/s (%.1f s)" % (head.name, v * 1e3, time.time() - t))
+
+    per = []
+    for w in workloads[1:]:
+        hot_ms, cold_ms = measure_secondary(stream, w, rounds=50)
+        rf = roofline(w, hot_ms)
+        entry_ = {"name": w.name, "workload": w.describe, "kernel": w.kernel, "dtype": w.dtype,
+                  "ms_per_launch": round(hot_ms, 5), "ms_per_launch_cache_flushed": round(cold_ms, 5),
+                  "roofline": rf, "roofline_cache_flushed": roofline(w, cold_ms)}
+        log("%s: %.4f ms (%.1f %s, %.1f%% of peak); cache-flushed %.4f ms (%.1f%%)" % (
+            w.name, hot_ms, rf["achieved"], rf["unit"], 100 * rf["frac"], cold_ms,
+            100 * entry_["roofline_cache_flushed"]["frac"]))
+        if not args.no_cpu and w.cpu:
+            t = time.time()
+            v, sample = w.cpu()
+            entry_["cpu_baseline"] = {"value": round(v, 6), "unit": w.unit, "cores": 1, "kind": "port", "sample": sample}
+            log("cpu baseline %s: %.4f %s (%.1f s)" % (w.name, v, w.unit, time.time() - t))
+        per.append(entry_)
+    result["per_config"] = per
+
+    for w in workloads:
+        for p in w.buffers:
+            stream.free(p)
+    stream.close()
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,52 @@
+// Shared device helpers for the gfx950 kernels: 128-bit vector types, bit
+// casts, wavefront-64 reductions and 16-bit float conversions.
+#ifndef IMEX_HIP_DEVICE_COMMON_H
+#define IMEX_HIP_DEVICE_COMMON_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace imexhip {
+
+constexpr int kWave = 64;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+// f16 / bf16 bits -> f32 (exact) and f32 -> 16-bit with round-to-nearest-even.
+__device__ __forceinline__ float half_bits_to_float(uint32_t h16) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h16)));
+}
+__device__ __forceinline__ uint32_t float_to_half_bits(float f) {
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b16) { return u2f(b16 << 16); }
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
+  uint32_t u = f2u(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u)
+    return (u & 0x80000000u) ? 0xffc0u : 0x7fc0u;
+  u += ((u >> 16) & 1u) + 0x7fffu;
+  return u >> 16;
+}
+
+// Butterfly reductions across the 64 lanes of a wavefront.  The xor shuffles
+// lower to DPP row operations for distances < 16 and to lane permutes above.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1)
+    v += __shfl_xor(v, off, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1)
+    v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+} // namespace imexhip
+#endif

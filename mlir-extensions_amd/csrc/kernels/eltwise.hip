@@ -1,0 +1,180 @@
+// Element-wise kernels: ReLU (f32 / f16 / bf16) and SiLU (f32).
+//
+// Reference op bodies: benchmarks/relu/relu_gpu.mlir.in:3-13 (cmpf ugt + select)
+// and benchmarks/silu/silu_gpu.mlir.in:3-19 (negf, exp, addf, divf, then mulf in
+// a second pass over a full-size temporary).  Here each is ONE streaming pass:
+// 128-bit loads and stores, four of them in flight per lane, HBM-bound.
+//
+// Kernel arguments follow the IMEX launch convention: one raw base pointer per
+// memref, scalars (index = i64) by value.
+//
+// Launch: block (256,1,1); grid (ceil(n / kElemsPerBlock), 1, 1).
+
+#include "device_common.h"
+
+using namespace imexhip;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kVecsPerThread = 4; // 4 x 16 B per lane in flight
+
+// ---------------------------------------------------------------------------
+// Generic streaming driver: Op works on one 16-byte vector (u32x4) and on one
+// scalar element (for ragged tails and unaligned bases).
+// ---------------------------------------------------------------------------
+template <typename Op, int kElemBytes>
+__device__ __forceinline__ void stream_map(const void *__restrict__ in, void *__restrict__ out, int64_t n,
+                                           Op op) {
+  constexpr int kElemsPerVec = 16 / kElemBytes;
+  constexpr int64_t kElemsPerBlock = int64_t(kThreads) * kVecsPerThread * kElemsPerVec;
+  const int64_t base = int64_t(blockIdx.x) * kElemsPerBlock;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  if (aligned && base + kElemsPerBlock <= n) {
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(in) + base * kElemBytes);
+    u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + base * kElemBytes);
+    u32x4 v[kVecsPerThread];
+#pragma unroll
+    for (int j = 0; j < kVecsPerThread; ++j)
+      v[j] = __builtin_nontemporal_load(src + j * kThreads + threadIdx.x);
+#pragma unroll
+    for (int j = 0; j < kVecsPerThread; ++j)
+      __builtin_nontemporal_store(op.vec(v[j]), dst + j * kThreads + threadIdx.x);
+  } else {
+    for (int64_t i = base + threadIdx.x; i < base + kElemsPerBlock && i < n; i += kThreads)
+      op.scalar(in, out, i);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// ReLU.  "ugt" = unordered or greater than: x if x > 0 or x is NaN (payload
+// kept), else the constant +0.0 (so -0.0 -> +0.0).  Done on the bit patterns,
+// which makes the result independent of the FP mode registers.
+// ---------------------------------------------------------------------------
+struct ReluF32 {
+  static __device__ __forceinline__ uint32_t one(uint32_t u) {
+    const bool keep = (static_cast<int32_t>(u) > 0) || (u > 0xff800000u);
+    return keep ? u : 0u;
+  }
+  __device__ __forceinline__ u32x4 vec(u32x4 v) const {
+    return u32x4{one(v.x), one(v.y), one(v.z), one(v.w)};
+  }
+  __device__ __forceinline__ void scalar(const void *in, void *out, int64_t i) const {
+    static_cast<uint32_t *>(out)[i] = one(static_cast<const uint32_t *>(in)[i]);
+  }
+};
+
+// 16-bit variants; kNanAbove = magnitude bits of +Inf (0x7c00 f16, 0x7f80 bf16).
+template <uint32_t kNanAbove> struct Relu16 {
+  static __device__ __forceinline__ uint32_t one(uint32_t h) {
+    const uint32_t mag = h & 0x7fffu;
+    const bool positive = (h & 0x8000u) == 0 && mag != 0;
+    const bool nan = mag > kNanAbove;
+    return (positive || nan) ? h : 0u;
+  }
+  static __device__ __forceinline__ uint32_t pair(uint32_t w) { return one(w & 0xffffu) | (one(w >> 16) << 16); }
+  __device__ __forceinline__ u32x4 vec(u32x4 v) const {
+    return u32x4{pair(v.x), pair(v.y), pair(v.z), pair(v.w)};
+  }
+  __device__ __forceinline__ void scalar(const void *in, void *out, int64_t i) const {
+    static_cast<uint16_t *>(out)[i] = static_cast<uint16_t>(one(static_cast<const uint16_t *>(in)[i]));
+  }
+};
+
+// ---------------------------------------------------------------------------
+// SiLU, f32, bit-compatible with the reference's CPU lowering: five separately
+// rounded f32 operations  t = -x; e = exp(t); d = e + 1; s = 1 / d; y = s * x
+// where exp is libm's expf (benchmarks/pipelines/linalg-to-cpu.pp:18-19).
+//
+// expf_libm restates the algorithm glibc's expf uses (Arm Optimized Routines
+// exp2f/expf: reduce x*32/ln2 = k + r, 2^(k/32) from a 32-entry table, cubic in
+// r, everything in f64, one final rounding to f32).  Every f64 operation here
+// is an IEEE one, so the result equals the host's for every input.
+// ---------------------------------------------------------------------------
+__device__ const uint64_t kExp2Table[32] = {
+    0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
+    0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
+    0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
+    0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,
+    0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
+    0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
+    0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
+    0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
+
+__device__ __forceinline__ float expf_libm(float x, const uint64_t *table) {
+  const uint32_t ux = f2u(x);
+  const uint32_t abstop = (ux >> 20) & 0x7ffu;
+  if (abstop >= 0x42bu) { // |x| >= 88 or NaN
+    if (ux == 0xff800000u)
+      return 0.0f;
+    if (abstop >= 0x7f8u)
+      return x + x;
+    if (x > 0x1.62e42ep6f)
+      return __builtin_inff();
+    if (x < -0x1.9fe368p6f)
+      return 0.0f;
+  }
+  constexpr double kInvLn2N = 0x1.71547652b82fep+0 * 32;
+  constexpr double kShift = 0x1.8p+52;
+  constexpr double kC0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32;
+  constexpr double kC1 = 0x1.ebfce50fac4f3p-3 / 32 / 32;
+  constexpr double kC2 = 0x1.62e42ff0c52d6p-1 / 32;
+  const double xd = static_cast<double>(x);
+  const double z = kInvLn2N * xd;
+  double kd = z + kShift;
+  const uint64_t ki = __builtin_bit_cast(uint64_t, kd);
+  kd -= kShift;
+  const double r = z - kd;
+  uint64_t t = table[ki & 31u];
+  t += ki << (52 - 5);
+  const double s = __builtin_bit_cast(double, t);
+  const double p = kC0 * r + kC1;
+  const double r2 = r * r;
+  double y = kC2 * r + 1.0;
+  y = p * r2 + y;
+  y = y * s;
+  return static_cast<float>(y);
+}
+
+struct SiluF32 {
+  const uint64_t *table;
+  __device__ __forceinline__ float one(float x) const {
+    const float t = -x;
+    const float e = expf_libm(t, table);
+    const float d = e + 1.0f;
+    const float s = 1.0f / d; // correctly rounded IEEE division
+    return s * x;
+  }
+  __device__ __forceinline__ u32x4 vec(u32x4 v) const {
+    return u32x4{f2u(one(u2f(v.x))), f2u(one(u2f(v.y))), f2u(one(u2f(v.z))), f2u(one(u2f(v.w)))};
+  }
+  __device__ __forceinline__ void scalar(const void *in, void *out, int64_t i) const {
+    static_cast<float *>(out)[i] = one(static_cast<const float *>(in)[i]);
+  }
+};
+
+} // namespace
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_relu_f32(const float *in, float *out, int64_t n) {
+  stream_map<ReluF32, 4>(in, out, n, ReluF32{});
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_relu_f16(const uint16_t *in, uint16_t *out,
+                                                                    int64_t n) {
+  stream_map<Relu16<0x7c00u>, 2>(in, out, n, Relu16<0x7c00u>{});
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_relu_bf16(const uint16_t *in, uint16_t *out,
+                                                                     int64_t n) {
+  stream_map<Relu16<0x7f80u>, 2>(in, out, n, Relu16<0x7f80u>{});
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_silu_f32(const float *in, float *out, int64_t n) {
+  // The 32-entry table is staged in LDS: the index is data-dependent, and LDS
+  // serves 64 different addresses per access where a constant load would not.
+  __shared__ uint64_t table[32];
+  if (threadIdx.x < 32)
+    table[threadIdx.x] = kExp2Table[threadIdx.x];
+  __syncthreads();
+  stream_map<SiluF32, 4>(in, out, n, SiluF32{table});
+}

@@ -1,0 +1,124 @@
+// Sum reductions, f32.
+//
+//  * imex_rowsum_f32: out[r] = init + sum_c in[r, c]  (row-sum / last-dim form:
+//    test/Integration/Dialect/XeGPU/WG/reduction_2D_1D_cross_sg_cross_lane.mlir:31-37,
+//    benchmarks/kInputFusion/kInputFusion.mlir.in:29-39).
+//    The reference's linalg path runs the whole sum in one work-item
+//    (test/SPIRV/OpTest.Sum_FLOAT32.mlir:39); here a workgroup (or a wavefront,
+//    for short rows) owns a row, streams it once with 128-bit loads, and
+//    combines partial sums with wavefront-64 butterflies and one LDS hop.
+//  * imex_reduce_outer_f32: out[i] = init + sum_o in[o, i], the OUTERMOST
+//    dimension reduced (benchmarks/reduce/reduce_gpu.mlir.in:4-21).  Each lane
+//    owns four adjacent outputs and adds the `outer` slices in order, which is
+//    the reference's summation order, so this one is bit-exact.
+//
+// Arguments: rowsum (in, out, rows: i64, cols: i64, init: f32);
+//            reduce_outer (in, out, outer: i64, inner: i64, init: f32).
+// Launch: block (256,1,1);
+//   rowsum: cols > 2048 -> grid (rows,1,1) [workgroup per row],
+//           else grid (ceil(rows/4),1,1)  [wavefront per row];
+//   reduce_outer: grid (ceil(inner / 1024), 1, 1).
+
+#include "device_common.h"
+
+using namespace imexhip;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWavesPerBlock = kThreads / kWave;
+constexpr int64_t kWavePerRowMaxCols = 2048;
+
+// Partial sum of one row over the lanes [tid, tid+stride, ...).
+__device__ __forceinline__ float row_partial(const float *__restrict__ row, int64_t cols, int tid, int stride) {
+  float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    const int64_t vecs = cols / 4;
+    const f32x4 *src = reinterpret_cast<const f32x4 *>(row);
+    int64_t v = tid;
+    // four independent 16-byte loads in flight per lane
+    for (; v + 3 * int64_t(stride) < vecs; v += 4 * int64_t(stride)) {
+      f32x4 a = __builtin_nontemporal_load(src + v);
+      f32x4 b = __builtin_nontemporal_load(src + v + stride);
+      f32x4 c = __builtin_nontemporal_load(src + v + 2 * int64_t(stride));
+      f32x4 d = __builtin_nontemporal_load(src + v + 3 * int64_t(stride));
+      acc[0] += (a.x + a.y) + (a.z + a.w);
+      acc[1] += (b.x + b.y) + (b.z + b.w);
+      acc[2] += (c.x + c.y) + (c.z + c.w);
+      acc[3] += (d.x + d.y) + (d.z + d.w);
+    }
+    for (; v < vecs; v += stride) {
+      f32x4 a = __builtin_nontemporal_load(src + v);
+      acc[0] += (a.x + a.y) + (a.z + a.w);
+    }
+    for (int64_t c = vecs * 4 + tid; c < cols; c += stride)
+      acc[1] += row[c];
+  } else {
+    for (int64_t c = tid; c < cols; c += stride)
+      acc[0] += row[c];
+  }
+  return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+}
+
+} // namespace
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_rowsum_f32(const float *in, float *out, int64_t rows,
+                                                                      int64_t cols, float init) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  if (cols > kWavePerRowMaxCols) {
+    __shared__ float partial[kWavesPerBlock];
+    const int64_t row = blockIdx.x;
+    if (row >= rows)
+      return;
+    float s = wave_sum(row_partial(in + row * cols, cols, threadIdx.x, kThreads));
+    if (lane == 0)
+      partial[wave] = s;
+    __syncthreads();
+    if (threadIdx.x == 0)
+      out[row] = init + ((partial[0] + partial[1]) + (partial[2] + partial[3]));
+  } else {
+    const int64_t row = int64_t(blockIdx.x) * kWavesPerBlock + wave;
+    if (row >= rows)
+      return;
+    float s = wave_sum(row_partial(in + row * cols, cols, lane, kWave));
+    if (lane == 0)
+      out[row] = init + s;
+  }
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_reduce_outer_f32(const float *in, float *out,
+                                                                            int64_t outer, int64_t inner,
+                                                                            float init) {
+  const int64_t i0 = (int64_t(blockIdx.x) * kThreads + threadIdx.x) * 4;
+  if (i0 >= inner)
+    return;
+  const bool vec = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
+                   (inner % 4) == 0;
+  if (vec) {
+    f32x4 acc = {init, init, init, init};
+    const f32x4 *src = reinterpret_cast<const f32x4 *>(in + i0);
+    const int64_t strideVecs = inner / 4;
+    int64_t o = 0;
+    for (; o + 4 <= outer; o += 4) { // loads issued together, adds kept in order
+      f32x4 a = __builtin_nontemporal_load(src + (o + 0) * strideVecs);
+      f32x4 b = __builtin_nontemporal_load(src + (o + 1) * strideVecs);
+      f32x4 c = __builtin_nontemporal_load(src + (o + 2) * strideVecs);
+      f32x4 d = __builtin_nontemporal_load(src + (o + 3) * strideVecs);
+      acc = acc + a;
+      acc = acc + b;
+      acc = acc + c;
+      acc = acc + d;
+    }
+    for (; o < outer; ++o)
+      acc = acc + __builtin_nontemporal_load(src + o * strideVecs);
+    *reinterpret_cast<f32x4 *>(out + i0) = acc;
+  } else {
+    for (int64_t i = i0; i < i0 + 4 && i < inner; ++i) {
+      float acc = init;
+      for (int64_t o = 0; o < outer; ++o)
+        acc = acc + in[o * inner + i];
+      out[i] = acc;
+    }
+  }
+}

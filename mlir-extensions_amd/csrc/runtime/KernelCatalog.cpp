@@ -1,0 +1,163 @@
+//===- KernelCatalog.cpp - embedded gfx950 code objects + launch shapes ----===//
+//
+// Host-side table of the hand-written kernels: which embedded code object
+// holds each one and the grid/block it is launched with.  This plays the part
+// of the `gpu.binary` blob plus the `blocks in (...) threads in (...)` operands
+// that IMEX's lowering bakes into host code
+// (lib/Conversion/GPUXToLLVM/GPUXToLLVMPass.cpp:456-713).
+//
+//===----------------------------------------------------------------------===//
+
+#include "imex_hip_kernels.h"
+
+#include <cstring>
+
+// Blob symbols come from the assembler stub generated at build time
+// (one .incbin per code object).
+extern "C" {
+extern const unsigned char imex_blob_eltwise[], imex_blob_eltwise_end[];
+extern const unsigned char imex_blob_softmax[], imex_blob_softmax_end[];
+extern const unsigned char imex_blob_reduce[], imex_blob_reduce_end[];
+extern const unsigned char imex_blob_transpose[], imex_blob_transpose_end[];
+extern const unsigned char imex_blob_gemm[], imex_blob_gemm_end[];
+}
+
+namespace {
+
+enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm };
+enum class Shape { Eltwise32, Eltwise16, SoftmaxRows, RowSum, ReduceOuter, Transpose2D, Transpose3D, Gemm, GemmFixed4k };
+
+struct Entry {
+  const char *name;
+  const char *signature;
+  Module module;
+  Shape shape;
+  int ndims;
+};
+
+const Entry kEntries[] = {
+    {"imex_relu_f32", "(in: f32*, out: f32*, n: i64)", Module::Eltwise, Shape::Eltwise32, 1},
+    {"imex_relu_f16", "(in: f16*, out: f16*, n: i64)", Module::Eltwise, Shape::Eltwise16, 1},
+    {"imex_relu_bf16", "(in: bf16*, out: bf16*, n: i64)", Module::Eltwise, Shape::Eltwise16, 1},
+    {"imex_silu_f32", "(in: f32*, out: f32*, n: i64)", Module::Eltwise, Shape::Eltwise32, 1},
+    {"imex_softmax_f32", "(in: f32*, out: f32*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows, 2},
+    {"imex_softmax_f16", "(in: f16*, out: f16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows, 2},
+    {"imex_softmax_bf16", "(in: bf16*, out: bf16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows, 2},
+    {"imex_rowsum_f32", "(in: f32*, out: f32*, rows: i64, cols: i64, init: f32)", Module::Reduce, Shape::RowSum, 2},
+    {"imex_reduce_outer_f32", "(in: f32*, out: f32*, outer: i64, inner: i64, init: f32)", Module::Reduce,
+     Shape::ReduceOuter, 2},
+    {"imex_transpose2d_b32", "(in: b32*, out: b32*, rows: i64, cols: i64)", Module::Transpose, Shape::Transpose2D, 2},
+    {"imex_transpose2d_b16", "(in: b16*, out: b16*, rows: i64, cols: i64)", Module::Transpose, Shape::Transpose2D, 2},
+    {"imex_transpose3d_b32", "(in: b32*, out: b32*, d0: i64, d1: i64, d2: i64)", Module::Transpose,
+     Shape::Transpose3D, 3},
+    {"imex_transpose3d_b16", "(in: b16*, out: b16*, d0: i64, d1: i64, d2: i64)", Module::Transpose,
+     Shape::Transpose3D, 3},
+    {"imex_gemm_f16_f16_f32", "(A: f16*, B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
+    {"imex_gemm_f16_f16_f32_acc", "(A: f16*, B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
+    {"imex_gemm_bf16_bf16_f32", "(A: bf16*, B: bf16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
+    {"imex_gemm_bf16_bf16_f32_acc", "(A: bf16*, B: bf16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm,
+     Shape::Gemm, 3},
+    {"imex_gemm_f16_f16_f16", "(A: f16*, B: f16*, C: f16*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
+    {"imex_gemm_bf16_bias_silu_bf16", "(A: bf16*, B: bf16*, bias: f32*, out: bf16*, M: i64, N: i64, K: i64)",
+     Module::Gemm, Shape::Gemm, 3},
+    {"imex_gemm_4kx4kx4k_f16_f16_f32", "(A: f16*, B: f16*, C: f32*)", Module::Gemm, Shape::GemmFixed4k, 0},
+    {"imex_gemm_4kx4kx4k_f16_f16_f32_bias", "(bias: f32*, C: f32*, A: f16*, B: f16*)", Module::Gemm,
+     Shape::GemmFixed4k, 0},
+};
+constexpr int kEntryCount = sizeof(kEntries) / sizeof(kEntries[0]);
+
+const Entry *find(const char *name) {
+  if (!name)
+    return nullptr;
+  for (const Entry &e : kEntries)
+    if (strcmp(e.name, name) == 0)
+      return &e;
+  return nullptr;
+}
+
+size_t ceilDiv(int64_t a, int64_t b) { return static_cast<size_t>((a + b - 1) / b); }
+
+} // namespace
+
+extern "C" int imexHipKernelCount(void) { return kEntryCount; }
+
+extern "C" const char *imexHipKernelName(int index) {
+  return (index >= 0 && index < kEntryCount) ? kEntries[index].name : nullptr;
+}
+
+extern "C" const char *imexHipKernelSignature(int index) {
+  return (index >= 0 && index < kEntryCount) ? kEntries[index].signature : nullptr;
+}
+
+extern "C" const void *imexHipKernelModule(const char *kernel, size_t *size) {
+  const Entry *e = find(kernel);
+  if (!e)
+    return nullptr;
+  const unsigned char *begin = nullptr, *end = nullptr;
+  switch (e->module) {
+  case Module::Eltwise: begin = imex_blob_eltwise; end = imex_blob_eltwise_end; break;
+  case Module::Softmax: begin = imex_blob_softmax; end = imex_blob_softmax_end; break;
+  case Module::Reduce: begin = imex_blob_reduce; end = imex_blob_reduce_end; break;
+  case Module::Transpose: begin = imex_blob_transpose; end = imex_blob_transpose_end; break;
+  case Module::Gemm: begin = imex_blob_gemm; end = imex_blob_gemm_end; break;
+  }
+  if (size)
+    *size = static_cast<size_t>(end - begin);
+  return begin;
+}
+
+extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims, int ndims, size_t grid[3],
+                                        size_t block[3], size_t *sharedMemBytes) {
+  const Entry *e = find(kernel);
+  if (!e)
+    return -1;
+  if (ndims != e->ndims || (ndims > 0 && !dims))
+    return -2;
+  for (int i = 0; i < ndims; ++i)
+    if (dims[i] < 0 || dims[i] > (int64_t(1) << 40))
+      return -2;
+  grid[0] = grid[1] = grid[2] = 1;
+  block[0] = 256;
+  block[1] = block[2] = 1;
+  if (sharedMemBytes)
+    *sharedMemBytes = 0;
+  switch (e->shape) {
+  case Shape::Eltwise32: // 256 lanes x 4 vectors x 4 elements
+    grid[0] = ceilDiv(dims[0], 4096);
+    break;
+  case Shape::Eltwise16: // 256 lanes x 4 vectors x 8 elements
+    grid[0] = ceilDiv(dims[0], 8192);
+    break;
+  case Shape::SoftmaxRows: // one wavefront per row, four per workgroup
+    grid[0] = ceilDiv(dims[0], 4);
+    if (dims[1] == 0)
+      grid[0] = 0;
+    break;
+  case Shape::RowSum: // workgroup per row above 2048 columns, else wavefront per row
+    grid[0] = dims[1] > 2048 ? static_cast<size_t>(dims[0]) : ceilDiv(dims[0], 4);
+    break;
+  case Shape::ReduceOuter: // four outputs per lane
+    grid[0] = ceilDiv(dims[1], 1024);
+    break;
+  case Shape::Transpose2D:
+    grid[0] = ceilDiv(dims[1], 64);
+    grid[1] = ceilDiv(dims[0], 64);
+    break;
+  case Shape::Transpose3D:
+    grid[0] = ceilDiv(dims[2], 64);
+    grid[1] = ceilDiv(dims[0], 64);
+    grid[2] = static_cast<size_t>(dims[1]);
+    break;
+  case Shape::Gemm: {
+    const int64_t M = dims[0], N = dims[1], K = dims[2];
+    const bool tileable = M > 0 && N > 0 && K > 0 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0;
+    grid[0] = tileable ? static_cast<size_t>((M / 256) * (N / 256)) : ceilDiv(M * N, 256);
+    break;
+  }
+  case Shape::GemmFixed4k:
+    grid[0] = 256;
+    break;
+  }
+  // A grid component of 0 means there is nothing to launch.
+  return 0;
+}

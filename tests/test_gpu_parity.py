@@ -1,0 +1,334 @@
+"""GPU parity tests: every kernel, called through the gpu* C ABI, against the CPU
+oracle on the same seeded inputs; reference golden vectors; size-independent
+properties at the full benchmark shapes.
+
+Bars: bit-exact for relu / transpose / reduce_outer / integer GEMM; <= 1 ulp for
+SiLU (f32); |d| <= 1e-3 |ref| + 2^-24 for f16 softmax (2^-24 = one f16 subnormal
+step, the output type's absolute resolution) and 1e-3 relative for row sums;
+max|d| <= 5e-3 max|ref| for the GEMMs.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "reference_vectors.json")) as f:
+    GOLD = json.load(f)
+
+
+def arr(v, shape=None):
+    a = np.asarray(v, np.float32)
+    return a.reshape(shape) if shape else a
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+
+
+# =============================== ReLU =====================================
+def test_relu_golden_and_specials(host, orc, stream):
+    g = GOLD["relu_f32_4x5_spirv"]
+    assert np.array_equal(host.relu(stream, arr(g["input"], g["shape"])), arr(g["expected"], g["shape"]))
+    x = np.array([0x7fc00001, 0xffc12345, 0x80000000, 0, 1, 0x80000001, 0x7f800000, 0xff800000, 0x7f800001],
+                 np.uint32).view(np.float32)
+    assert np.array_equal(host.relu(stream, x).view(np.uint32), orc.relu_f32(x).view(np.uint32))
+
+
+@pytest.mark.parametrize("n", [1, 3, 4095, 4096, 4097, 100003, 1 << 20])
+def test_relu_ragged_sizes(host, orc, stream, n):
+    say("relu n=%d" % n)
+    x = orc.fill_uniform(n, "f32", 20241 + n % 7, -1.0, 1.0)
+    assert np.array_equal(host.relu(stream, x).view(np.uint32), orc.relu_f32(x).view(np.uint32))
+
+
+def test_relu_config_4096x4096(host, orc, stream):
+    x = orc.fill_uniform(4096 * 4096, "f32", 20241, -1.0, 1.0).reshape(4096, 4096)
+    assert np.array_equal(host.relu(stream, x).view(np.uint32), orc.relu_f32(x).view(np.uint32))
+
+
+def test_relu_every_f32_pattern(host, stream):
+    """All 2^32 bit patterns against the closed form (x if x > 0 or NaN else +0)."""
+    chunk = 1 << 27
+    for base in range(0, 1 << 32, chunk):
+        if base % (1 << 30) == 0:
+            say("relu sweep base=0x%08x" % base)
+        u = np.arange(base, base + chunk, dtype=np.uint32)
+        got = host.relu(stream, u.view(np.float32)).view(np.uint32)
+        keep = (u.view(np.int32) > 0) | (u > np.uint32(0xff800000))
+        assert np.array_equal(got, np.where(keep, u, np.uint32(0)))
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_relu_every_16bit_pattern(host, orc, stream, dtype):
+    x = np.tile(np.arange(65536, dtype=np.uint16), 3)[:-5]  # unaligned tail
+    assert np.array_equal(host.relu(stream, x, dtype), orc.relu_16(x, dtype))
+
+
+# =============================== SiLU =====================================
+def test_silu_within_one_ulp(host, orc, stream):
+    x = np.concatenate([
+        orc.fill_uniform(1 << 20, "f32", 20251, -8.0, 8.0),
+        orc.fill_uniform(1 << 18, "f32", 1, -110.0, 110.0),
+        orc.fill_bits(1 << 18, "f32", 2).view(np.float32),
+        np.array([0.0, -0.0, 1.3, np.inf, -np.inf, 88.0, -88.0, 88.72, 88.73, -103.9, -104.0, 1e-45, -1e-45, 1e38,
+                  -1e38], np.float32),
+        np.array([0x7fc00000], np.uint32).view(np.float32)])
+    got, ref = host.silu(stream, x), orc.silu_f32(x)
+    nan = np.isnan(ref)
+    assert np.array_equal(np.isnan(got), nan)
+    d = orc.ulp_distance_f32(got[~nan], ref[~nan])
+    say("silu max ulp distance %d, exact %d of %d" % (d.max(), int((d == 0).sum()), d.size))
+    assert d.max() <= 1
+    assert host.silu(stream, np.array([0.0], np.float32))[0] == 0.0
+
+
+def test_silu_benchmark_shape(host, orc, stream):
+    x = orc.fill_uniform(512 * 640 * 20 * 15, "f32", 20251, -8.0, 8.0)
+    got, ref = host.silu(stream, x), orc.silu_f32(x)
+    assert orc.ulp_distance_f32(got, ref).max() <= 1
+
+
+# =============================== Softmax ==================================
+def close_16(orc, got_bits, ref_bits, dtype):
+    got, ref = orc.to_float(got_bits, dtype), orc.to_float(ref_bits, dtype)
+    quantum = 2.0 ** -24 if dtype == "f16" else 0.0
+    rtol = 1e-3 if dtype == "f16" else 2.0 ** -7  # bf16: one unit in the last place
+    return np.all(np.abs(got - ref) <= rtol * np.abs(ref) + quantum)
+
+
+@pytest.mark.parametrize("key", ["softmax_f32_10x20", "softmax_f32_10x20_spirv"])
+def test_softmax_golden(host, orc, stream, key):
+    g = GOLD[key]
+    got = host.softmax(stream, arr(g["input"], g["shape"]), "f32")
+    want = arr(g["expected"], g["shape"])
+    assert np.max(np.abs(got - want) / want) < 2e-5
+    assert orc.allclose_f32(got, want)
+
+
+def test_softmax_config_f16_16384x1024(host, orc, stream):
+    x = orc.fill_normal(16384 * 1024, "f16", 20242, 0.0, 2.0).reshape(16384, 1024)
+    got, ref = host.softmax(stream, x, "f16"), orc.softmax_16(x, "f16")
+    assert close_16(orc, got, ref, "f16")
+    assert orc.allclose_f32(orc.half_to_float(got), orc.softmax_f32(orc.half_to_float(x)))
+    sums = orc.half_to_float(got).sum(axis=1, dtype=np.float64)
+    assert np.max(np.abs(sums - 1.0)) < 2e-3  # 1024 outputs each rounded to f16
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 7), (5, 8), (16, 2000), (64, 2000), (7, 1000), (9, 512), (4, 4096),
+                                       (3, 5000), (2, 65536 + 8), (1025, 64), (6, 1016)])
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_softmax_shapes(host, orc, stream, rows, cols, dtype):
+    say("softmax %s %dx%d" % (dtype, rows, cols))
+    x = orc.fill_normal(rows * cols, dtype, rows * 131 + cols, 0.0, 2.0).reshape(rows, cols)
+    got = host.softmax(stream, x, dtype)
+    if dtype == "f32":
+        ref = orc.softmax_f32(x)
+        assert np.all(np.abs(got - ref) <= 1e-3 * np.abs(ref))
+        assert np.max(np.abs(got - ref) / np.maximum(ref, 1e-30)) < 5e-5
+    else:
+        assert close_16(orc, got, orc.softmax_16(x, "f16"), "f16")
+
+
+def test_softmax_bf16_and_exact_rows(host, orc, stream):
+    x = orc.fill_normal(64 * 1024, "bf16", 9, 0.0, 2.0).reshape(64, 1024)
+    assert close_16(orc, host.softmax(stream, x, "bf16"), orc.softmax_16(x, "bf16"), "bf16")
+    eq = orc.float_to_half(np.full((8, 1024), 3.3, np.float32))
+    assert np.all(host.softmax(stream, eq, "f16") == 0x1400)  # exactly 2^-10
+    # a row of -inf-free extremes: one dominant element
+    x = np.full((4, 1024), -20.0, np.float32)
+    x[:, 5] = 20.0
+    got = host.softmax(stream, x, "f32")
+    assert np.all(got[:, 5] == 1.0) and got.sum() == 4.0
+
+
+# =============================== Reductions ================================
+def test_rowsum_golden_and_exact(host, orc, stream):
+    g = GOLD["sum_f32_10x20"]
+    x = arr(g["input"], g["shape"])
+    assert np.array_equal(host.rowsum(stream, x), np.full(10, 210.0, np.float32))
+    assert host.rowsum(stream, x.reshape(1, 200))[0] == 2100.0
+    g = GOLD["wg_reduction_rows"]
+    x = np.repeat(np.arange(8, dtype=np.float32)[:, None], 256, axis=1)
+    assert list(host.rowsum(stream, x)) == g["expected"]
+    assert host.rowsum(stream, np.ones((1, 65536), np.float32))[0] == 65536.0
+    # integer-valued inputs: any summation order is exact
+    for rows, cols in [(37, 1000), (5, 8192), (3, 4099), (130, 2048), (2, 2052), (9, 1)]:
+        xi = orc.fill_int(rows * cols, "f32", rows + cols, -8, 8).reshape(rows, cols)
+        assert np.array_equal(host.rowsum(stream, xi, init=3.0), orc.rowsum_f32(xi, init=3.0)), (rows, cols)
+
+
+def test_rowsum_config_8192x8192(host, orc, stream):
+    x = orc.fill_uniform(8192 * 8192, "f32", 20243, 0.0, 1.0).reshape(8192, 8192)
+    got, ref = host.rowsum(stream, x), orc.rowsum_f32(x)
+    assert np.max(np.abs(got - ref) / np.abs(ref)) <= 1e-3
+    exact = x.sum(axis=1, dtype=np.float64)
+    say("rowsum rel err vs f64: kernel %.2e, sequential oracle %.2e" %
+        (np.max(np.abs(got - exact) / exact), np.max(np.abs(ref - exact) / exact)))
+    assert np.max(np.abs(got - exact) / exact) < 1e-5
+
+
+@pytest.mark.parametrize("shape", [(32, 16, 64, 64), (10, 20), (7, 1023), (33, 4100), (1, 5), (3, 1, 9)])
+def test_reduce_outer_bit_exact(host, orc, stream, shape):
+    x = orc.fill_uniform(int(np.prod(shape)), "f32", 77, -1.0, 1.0).reshape(shape)
+    got, ref = host.reduce_outer(stream, x, init=0.25), orc.reduce_outer_f32(x, init=0.25)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+
+
+# =============================== Transpose =================================
+def test_transpose_golden(host, orc, stream):
+    g = GOLD["transpose_f32_10x20"]
+    assert np.array_equal(host.transpose2d(stream, arr(g["input"], g["shape"])), arr(g["expected"], [20, 10]))
+    g = GOLD["transpose_bf16_10x20"]
+    xb = orc.float_to_bfloat(arr(g["input"], g["shape"]))
+    assert np.array_equal(orc.bfloat_to_float(host.transpose2d(stream, xb)), arr(g["expected"], [20, 10]))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (64, 64), (128, 136), (1024, 1024), (63, 65), (8, 2000), (200, 8),
+                                       (72, 520), (1000, 3), (257, 129)])
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_transpose_shapes_bit_exact(host, orc, stream, rows, cols, dtype):
+    say("transpose %s %dx%d" % (dtype, rows, cols))
+    x = orc.fill_bits(rows * cols, dtype, 20244 + rows).reshape(rows, cols)
+    got = host.transpose2d(stream, x)
+    assert np.array_equal(got, orc.transpose2d(x))
+    assert np.array_equal(host.transpose2d(stream, got), x)  # involution
+
+
+def test_transpose_config_sizes(host, orc, stream):
+    x = orc.fill_bits(8192 * 8192, "bf16", 20244).reshape(8192, 8192)
+    got = host.transpose2d(stream, x)
+    assert np.array_equal(got, x.T)
+    # index-encoded input: every element lands where its index says
+    idx = np.arange(4096 * 4096, dtype=np.uint32).reshape(4096, 4096)
+    assert np.array_equal(host.transpose2d(stream, idx), idx.T)
+    y = orc.fill_bits(4096 * 4096, "f32", 20245).reshape(4096, 4096)
+    assert np.array_equal(host.transpose2d(stream, y), orc.transpose2d(y))
+
+
+@pytest.mark.parametrize("shape", [(16, 96, 96), (96, 7, 96), (5, 3, 9), (64, 2, 72)])
+def test_transpose3d(host, orc, stream, shape):
+    n = int(np.prod(shape))
+    x32 = orc.fill_bits(n, "f32", 5).reshape(shape)
+    assert np.array_equal(host.transpose3d(stream, x32), orc.transpose3d(x32))
+    x16 = orc.fill_bits(n, "f16", 6).reshape(shape)
+    assert np.array_equal(host.transpose3d(stream, x16), x16.transpose(2, 1, 0))
+
+
+# =============================== GEMM ======================================
+def gemm_close(got, ref):
+    return np.max(np.abs(got - ref)) <= 5e-3 * np.max(np.abs(ref))
+
+
+def test_gemm_golden_3x3(host, orc, stream):
+    g = GOLD["gemm_f16_acc_f32_3x3"]
+    a, b = orc.float_to_half(arr(g["A"], [3, 3])), orc.float_to_half(arr(g["B"], [3, 3]))
+    c = host.gemm(stream, a, b, c=arr(g["C0"], [3, 3]), ab_dtype="f16")
+    assert orc.allclose_f32(c, arr(g["expected"], [3, 3]))
+    assert np.array_equal(c, orc.gemm(a, b, "f16", c=arr(g["C0"], [3, 3])))  # scalar path: same order, bit-exact
+    g = GOLD["gemm_bf16_acc_f32_3x3"]
+    a, b = orc.float_to_bfloat(arr(g["A"], [3, 3])), orc.float_to_bfloat(arr(g["B"], [3, 3]))
+    c = host.gemm(stream, a, b, c=arr(g["C0"], [3, 3]), ab_dtype="bf16")
+    assert np.max(np.abs(c.ravel() - arr(g["expected"]))) < 6e-5
+    g = GOLD["dot_f16_acc_f32_8x16x32"]
+    a = orc.float_to_half(np.full((8, 16), 1.0, np.float32))
+    b = orc.float_to_half(np.full((16, 32), 2.0, np.float32))
+    out = host.gemm(stream, a, b, ab_dtype="f16", out_dtype="f16")
+    assert np.all(orc.half_to_float(out) == g["expected_fill"])
+
+
+@pytest.mark.parametrize("M,N,K", [(5, 7, 9), (100, 36, 130), (256, 256, 32), (255, 256, 64), (17, 300, 64)])
+def test_gemm_untileable_shapes_bit_exact(host, orc, stream, M, N, K):
+    a = orc.fill_uniform(M * K, "f16", 1, -1, 1).reshape(M, K)
+    b = orc.fill_uniform(K * N, "f16", 2, -1, 1).reshape(K, N)
+    assert np.array_equal(host.gemm(stream, a, b, ab_dtype="f16"), orc.gemm(a, b, "f16"))
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_tiled_identity_and_layout(host, orc, stream, dtype):
+    """B = I gives C = A exactly; A[i,j] = j patterns expose any fragment-layout mistake."""
+    M, N, K = 512, 512, 512
+    a = orc.fill_uniform(M * K, dtype, 3, -1, 1).reshape(M, K)
+    eye = orc.from_float(np.eye(K, dtype=np.float32), dtype)
+    assert np.array_equal(host.gemm(stream, a, eye, ab_dtype=dtype), orc.to_float(a, dtype))
+    # A = I: C = B exactly (exercises the B transpose-in-registers path)
+    b = orc.fill_uniform(K * N, dtype, 4, -1, 1).reshape(K, N)
+    assert np.array_equal(host.gemm(stream, eye, b, ab_dtype=dtype), orc.to_float(b, dtype))
+    # a single non-zero k picks out one row of B scaled by a column of A
+    a1 = np.zeros((M, K), np.float32)
+    a1[:, 77] = np.arange(M) % 16
+    got = host.gemm(stream, orc.from_float(a1, dtype), b, ab_dtype=dtype)
+    assert np.array_equal(got, np.outer(a1[:, 77], orc.to_float(b, dtype)[77]).astype(np.float32))
+
+
+@pytest.mark.parametrize("dtype,M,N,K", [("f16", 512, 768, 4096), ("bf16", 256, 1024, 1024), ("f16", 1024, 256, 64)])
+def test_gemm_tiled_small_integers_exact(host, orc, stream, dtype, M, N, K):
+    """|a|,|b| <= 4: every partial sum is an integer below 2^24, so any
+    accumulation order gives the same f32 bits as the integer product."""
+    a = orc.fill_int(M * K, dtype, 5, -4, 4).reshape(M, K)
+    b = orc.fill_int(K * N, dtype, 6, -4, 4).reshape(K, N)
+    want = orc.to_float(a, dtype).astype(np.int64) @ orc.to_float(b, dtype).astype(np.int64)
+    got = host.gemm(stream, a, b, ab_dtype=dtype)
+    assert np.array_equal(got.astype(np.int64), want)
+
+
+def test_gemm_config_f16_4096(host, orc, stream):
+    M = N = K = 4096
+    a = orc.fill_uniform(M * K, "f16", 20246, -1, 1).reshape(M, K)
+    b = orc.fill_uniform(K * N, "f16", 20247, -1, 1).reshape(K, N)
+    got = host.gemm(stream, a, b, ab_dtype="f16")
+    rows = np.array(sorted(set(list(range(0, 4096, 97)) + [1, 255, 256, 2047, 4095])))
+    ref = orc.gemm_rows(a, b, rows, "f16")
+    err = np.max(np.abs(got[rows] - ref)) / np.max(np.abs(ref))
+    say("gemm f16 4096^3: max|d|/max|ref| = %.3e over %d rows" % (err, rows.size))
+    assert err <= 5e-3
+    # the remaining rows: linearity / checksum  (1^T C) == (1^T A) B in f64
+    colsum = got.sum(axis=0, dtype=np.float64)
+    want = orc.half_to_float(a).sum(axis=0, dtype=np.float64) @ orc.half_to_float(b).astype(np.float64)
+    assert np.max(np.abs(colsum - want)) <= 1e-3 * np.max(np.abs(want)) + 0.05
+    # accumulate variant and the reference-signature entry point give C0 + A.B
+    c0 = orc.fill_uniform(M * N, "f32", 1, -1, 1).reshape(M, N)
+    acc = host.gemm(stream, a, b, c=c0, ab_dtype="f16")
+    assert np.max(np.abs(acc - (c0 + got))) <= 1e-4
+    d_a, d_b, d_c = stream.to_device(a), stream.to_device(b), stream.to_device(c0)
+    fn = stream.kernel("imex_gemm_4kx4kx4k_f16_f16_f32")
+    descs, keep = host._pack_params([d_a, d_b, d_c])
+    import ctypes as C
+    stream.rt.gpuLaunchKernel(stream.handle, fn, 16, 16, 1, 256, 1, 1, 0, C.cast(descs, C.c_void_p), None)
+    stream.wait()
+    fixed = stream.from_device(d_c, (M, N), np.float32)
+    for p in (d_a, d_b, d_c):
+        stream.free(p)
+    assert np.array_equal(fixed, acc)
+
+
+def test_gemm_config_mlp_bf16_bias_silu(host, orc, stream):
+    M, K, N = 4096, 4096, 11008
+    a = orc.fill_normal(M * K, "bf16", 20248, 0.0, 1.0).reshape(M, K)
+    b = orc.fill_normal(K * N, "bf16", 20249, 0.0, 0.02).reshape(K, N)
+    bias = orc.fill_normal(N, "f32", 20250, 0.0, 0.1)
+    got = orc.bfloat_to_float(host.gemm_bias_silu(stream, a, b, bias))
+    rows = np.array([0, 1, 255, 256, 1000, 2047, 2048, 3333, 4095])
+    ref = orc.bfloat_to_float(orc.bias_silu_bf16(orc.gemm_rows(a, b, rows, "bf16"), bias))
+    err = np.max(np.abs(got[rows] - ref)) / np.max(np.abs(ref))
+    say("mlp gemm: max|d|/max|ref| = %.3e" % err)
+    assert err <= 5e-3
+    # element-wise: within one bf16 step wherever the value is not tiny
+    big = np.abs(ref) > 1e-2
+    assert np.max(np.abs(got[rows][big] - ref[big]) / np.abs(ref[big])) <= 2.0 ** -7
+    # plain bf16 GEMM with f32 output against the same rows
+    plain = host.gemm(stream, a, b, ab_dtype="bf16")
+    ref32 = orc.gemm_rows(a, b, rows, "bf16")
+    assert gemm_close(plain[rows], ref32)
+
+
+def test_gemm_f16_output_variant(host, orc, stream):
+    M, N, K = 512, 256, 256
+    a = orc.fill_uniform(M * K, "f16", 8, -1, 1).reshape(M, K)
+    b = orc.fill_uniform(K * N, "f16", 9, -1, 1).reshape(K, N)
+    got = orc.half_to_float(host.gemm(stream, a, b, ab_dtype="f16", out_dtype="f16"))
+    ref = orc.gemm(a, b, "f16", out_round="f16")
+    assert gemm_close(got, ref)

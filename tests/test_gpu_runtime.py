@@ -1,0 +1,153 @@
+"""GPU tests of the runtime-wrapper ABI itself: allocation kinds, copies in every
+direction, module/kernel caching, event dependencies, the profiling loop and the
+upstream mgpu* entry points."""
+import ctypes as C
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_shared_allocation_is_host_dereferenceable(host, orc, stream):
+    n = 4096 + 5
+    p_in = stream.alloc(n * 4, shared=True)
+    p_out = stream.alloc(n * 4, shared=True)
+    assert int(p_in) % 256 == 0
+    x = orc.fill_uniform(n, "f32", 1, -1, 1)
+    # host code writes straight into the shared buffer, as JIT'd memref.copy does
+    C.memmove(int(p_in), x.ctypes.data, n * 4)
+    stream.launch("imex_relu_f32", [n], [p_in, p_out, n])
+    stream.wait()
+    got = np.ctypeslib.as_array(C.cast(int(p_out), C.POINTER(C.c_float)), shape=(n,)).copy()
+    assert np.array_equal(got, orc.relu_f32(x))
+    stream.free(p_in)
+    stream.free(p_out)
+
+
+def test_copies_in_every_direction(host, stream):
+    x = np.arange(100000, dtype=np.uint32)
+    d1, d2 = stream.alloc(x.nbytes), stream.alloc(x.nbytes)
+    stream.copy(d1, x.ctypes.data, x.nbytes)     # H2D
+    stream.copy(d2, d1, x.nbytes)                # D2D
+    y = np.zeros_like(x)
+    stream.copy(y.ctypes.data, d2, x.nbytes)     # D2H
+    z = np.zeros_like(x)
+    stream.copy(z.ctypes.data, y.ctypes.data, x.nbytes)  # H2H
+    assert np.array_equal(x, y) and np.array_equal(x, z)
+    stream.copy(d1, x.ctypes.data, 0)            # empty copy is a no-op
+    stream.free(d1)
+    stream.free(d2)
+
+
+def test_alignment_and_zero_size(host, stream):
+    p = stream.alloc(1000, alignment=4096)
+    assert int(p) % 4096 == 0
+    stream.free(p)
+    q = stream.alloc(0)
+    assert int(q) != 0
+    stream.free(q)
+
+
+def test_module_and_kernel_caching(host, stream):
+    rt, k = stream.rt, host.kernels()
+    size = C.c_size_t(0)
+    blob = k.imexHipKernelModule(b"imex_relu_f32", C.byref(size))
+    m1 = rt.gpuModuleLoad(stream.handle, blob, size.value)
+    m2 = rt.gpuModuleLoad(stream.handle, blob, size.value)
+    assert m1 == m2 and m1
+    f1 = rt.gpuKernelGet(stream.handle, m1, b"imex_relu_f32")
+    f2 = rt.gpuKernelGet(stream.handle, m1, b"imex_relu_f32")
+    assert f1 == f2 and f1
+    assert rt.gpuKernelGet(stream.handle, m1, b"imex_silu_f32") != f1
+
+
+def test_unknown_kernel_name_aborts_with_message():
+    prog = ("import sys; sys.path.insert(0, %r)\nimport __graft_entry__ as e\nhost = e.load_package().host\n"
+            "import ctypes as C\ns = host.Stream()\nsize = C.c_size_t(0)\n"
+            "blob = host.kernels().imexHipKernelModule(b'imex_relu_f32', C.byref(size))\n"
+            "m = s.rt.gpuModuleLoad(s.handle, blob, size.value)\ns.rt.gpuKernelGet(s.handle, m, b'no_such_kernel')\n" % REPO)
+    r = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert r.returncode == -6
+    assert "An exception was thrown: gpuKernelGet: kernel 'no_such_kernel' not found" in r.stdout
+
+
+def test_event_dependencies_across_streams(host, orc):
+    n = 1 << 20
+    x = orc.fill_uniform(n, "f32", 3, -1, 1)
+    with host.Stream() as s1, host.Stream() as s2:
+        d_in, d_mid, d_out = s1.to_device(x), s1.alloc(n * 4), s1.alloc(n * 4)
+        ev = s1.launch("imex_silu_f32", [n], [d_in, d_mid, n])
+        assert ev
+        # the second stream's launch waits on the first stream's event
+        s2.launch("imex_relu_f32", [n], [d_mid, d_out, n], deps=[ev])
+        s2.wait()
+        got = s2.from_device(d_out, (n,), np.float32)
+        assert np.array_equal(got, orc.relu_f32(orc.silu_f32(x)))
+        assert s1.elapsed_ms(ev, ev) == 0.0
+        for p in (d_in, d_mid, d_out):
+            s1.free(p)
+
+
+def test_profile_helper_modes(host, orc, stream):
+    n = 1 << 22
+    d_in, d_out = stream.to_device(orc.fill_uniform(n, "f32", 4, -1, 1)), stream.alloc(n * 4)
+    per_launch = stream.profile("imex_relu_f32", [n], [d_in, d_out, n], warmups=2, rounds=10, mode=0)
+    assert len(per_launch) == 10 and all(0 < t < 50 for t in per_launch)
+    flushed = stream.profile("imex_relu_f32", [n], [d_in, d_out, n], warmups=2, rounds=5, flush_bytes=64 << 20, mode=0)
+    assert len(flushed) == 5 and all(t > 0 for t in flushed)
+    total = stream.profile("imex_relu_f32", [n], [d_in, d_out, n], warmups=2, rounds=10, mode=1)
+    assert len(total) == 1 and 0 < total[0] < 500
+    stream.free(d_in)
+    stream.free(d_out)
+
+
+def test_profiling_env_prints_reference_line():
+    prog = ("import sys; sys.path.insert(0, %r)\nimport __graft_entry__ as e\nimport numpy as np\n"
+            "host = e.load_package().host\ns = host.Stream()\n"
+            "y = host.relu(s, np.linspace(-1, 1, 5000).astype(np.float32))\nprint('result', float(y.sum()))\n" % REPO)
+    env = dict(os.environ, IMEX_ENABLE_PROFILING="1", IMEX_PROFILING_RUNS="7", IMEX_PROFILING_WARMUPS="2",
+               IMEX_ENABLE_CACHE_FLUSHING="1", IMEX_CACHE_FLUSH_BYTES=str(32 << 20))
+    r = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                       timeout=300, env=env)
+    assert r.returncode == 0, r.stdout + r.stderr
+    line = [l for l in r.stdout.splitlines() if "execution time" in l]
+    assert len(line) == 1
+    assert line[0].startswith("the kernel execution time is (ms, on HIP runtime):avg: ")
+    assert line[0].endswith("(over 7 runs)")
+    for key in ("min:", "max:", "median:", "std_deviation:", "variance:", "P95:", "P5:", "median_one_third_avg:"):
+        assert key in line[0]
+    assert "result" in r.stdout  # the real launch still happens after profiling
+
+
+def test_mgpu_entry_points(host, orc):
+    rt, k = host.runtime(), host.kernels()
+    n = 10000
+    x = orc.fill_uniform(n, "f32", 5, -1, 1)
+    s = rt.mgpuStreamCreate()
+    d_in = rt.mgpuMemAlloc(n * 4, s, 0)
+    d_out = rt.mgpuMemAlloc(n * 4, s, 0)
+    rt.mgpuMemcpy(d_in, x.ctypes.data, n * 4, s)
+    rt.mgpuMemset32(d_out, 0x3f800000, n, s)
+    size = C.c_size_t(0)
+    blob = k.imexHipKernelModule(b"imex_relu_f32", C.byref(size))
+    fn = rt.mgpuModuleGetFunction(rt.mgpuModuleLoad(blob, size.value), b"imex_relu_f32")
+    args = [C.c_void_p(d_in), C.c_void_p(d_out), C.c_int64(n)]
+    argv = (C.c_void_p * 3)(*[C.cast(C.pointer(a), C.c_void_p) for a in args])
+    grid, block, _ = host.launch_shape("imex_relu_f32", [n])
+    ones = np.zeros(n, np.float32)
+    rt.mgpuStreamSynchronize(s)
+    rt.mgpuMemcpy(ones.ctypes.data, d_out, n * 4, s)
+    assert np.all(ones == 1.0)
+    rt.mgpuLaunchKernel(fn, grid[0], 1, 1, block[0], 1, 1, 0, s, argv, None, 3)
+    rt.mgpuStreamSynchronize(s)
+    y = np.zeros(n, np.float32)
+    rt.mgpuMemcpy(y.ctypes.data, d_out, n * 4, s)
+    assert np.array_equal(y, orc.relu_f32(x))
+    rt.mgpuMemFree(s, d_in)
+    rt.mgpuMemFree(s, d_out)
+    rt.mgpuStreamDestroy(s)

@@ -1,0 +1,333 @@
+"""Pins the CPU oracle: reference golden vectors, closed forms, exhaustive
+conversion checks, and the reference's own statistics code (oracle/_ref)."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "reference_vectors.json")) as f:
+    GOLD = json.load(f)
+
+
+def arr(v, shape=None):
+    a = np.asarray(v, np.float32)
+    return a.reshape(shape) if shape else a
+
+
+# ---- generators ---------------------------------------------------------------
+def test_mt19937_known_answer(orc):
+    # [rand.predef]: the 10000th consecutive invocation of a default-constructed
+    # std::mt19937 (seed 5489) produces 4123659995.
+    assert orc.mt19937_raw(5489, 10000)[-1] == 4123659995
+
+
+def test_uniform_matches_definition(orc):
+    raw = orc.mt19937_raw(20241, 64)
+    want = np.array([np.float32(-1.0 + 2.0 * ((w >> 8) / 16777216.0)) for w in raw], np.float32)
+    got = orc.fill_uniform(64, "f32", 20241, -1.0, 1.0)
+    assert np.array_equal(got, want)
+    assert got.min() >= -1.0 and got.max() < 1.0
+
+
+def test_normal_moments_and_definition(orc):
+    x = orc.fill_normal(200000, "f32", 20242, 0.0, 2.0)
+    assert abs(float(x.mean())) < 0.02 and abs(float(x.std()) - 2.0) < 0.02
+    w = orc.mt19937_raw(20242, 2)
+    u1, u2 = ((w[0] >> 8) + 1) / 16777216.0, (w[1] >> 8) / 16777216.0
+    r = math.sqrt(-2.0 * math.log(u1))
+    assert x[0] == np.float32(2.0 * r * math.cos(2 * math.pi * u2))
+    assert x[1] == np.float32(2.0 * r * math.sin(2 * math.pi * u2))
+
+
+def test_bits_have_no_nan(orc):
+    f = orc.fill_bits(100000, "f32", 20245).view(np.float32)
+    assert not np.isnan(f).any()
+    h = orc.fill_bits(100000, "f16", 1).view(np.float16)
+    assert not np.isnan(h).any()
+    b = orc.fill_bits(100000, "bf16", 20244)
+    assert not np.isnan(orc.bfloat_to_float(b)).any()
+    assert len(np.unique(b)) > 30000  # covers the 16-bit space, infinities included
+
+
+# ---- conversions ----------------------------------------------------------------
+def test_half_to_float_exhaustive(orc):
+    h = np.arange(65536, dtype=np.uint16)
+    got = orc.half_to_float(h)
+    want = h.view(np.float16).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_bfloat_to_float_exhaustive(orc):
+    b = np.arange(65536, dtype=np.uint16)
+    assert np.array_equal(orc.bfloat_to_float(b).view(np.uint32), b.astype(np.uint32) << 16)
+
+
+def test_float_to_half_rne(orc):
+    rng = np.random.default_rng(0)
+    bits = rng.integers(0, 2 ** 32, 2_000_000, dtype=np.uint64).astype(np.uint32)
+    # add every half value, every midpoint between adjacent halves, and neighbours
+    h = np.arange(0x7c00, dtype=np.uint16).view(np.float16).astype(np.float32)
+    mid = ((h[:-1].astype(np.float64) + h[1:].astype(np.float64)) / 2).astype(np.float32)
+    extra = np.concatenate([h, mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(np.inf)),
+                            -mid, np.array([65504, 65519.99, 65520, 1e9, np.inf, -np.inf, 0.0, -0.0], np.float32)])
+    f = np.concatenate([bits.view(np.float32), extra])
+    f = f[~np.isnan(f)]
+    with np.errstate(over="ignore"):
+        want = f.astype(np.float16).view(np.uint16)
+    assert np.array_equal(orc.float_to_half(f), want)
+    assert orc.float_to_half(np.array([np.nan], np.float32))[0] & 0x7fff == 0x7e00
+
+
+def test_float_to_bfloat_rne(orc):
+    rng = np.random.default_rng(1)
+    f = rng.integers(0, 2 ** 32, 1_000_000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    f = f[~np.isnan(f)]
+    u = f.view(np.uint32).astype(np.uint64)
+    want = ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    assert np.array_equal(orc.float_to_bfloat(f), want)
+    # values the reference's bf16 tests print after a round trip
+    # (OpTest.GEMM_BF16_ACC_F32.mlir:13: 1.999510e-01 -> bf16 -> contributes 14.1006)
+    assert orc.bfloat_to_float(orc.float_to_bfloat(np.array([0.199951], np.float32)))[0] == np.float32(0.2001953125)
+    # exact ties go to even
+    assert orc.float_to_bfloat(np.array([1.00390625], np.float32))[0] == 0x3f80
+    assert orc.float_to_bfloat(np.array([1.01171875], np.float32))[0] == 0x3f82
+
+
+# ---- relu ------------------------------------------------------------------------
+def test_relu_golden(orc):
+    g = GOLD["relu_f32_4x5_spirv"]
+    assert np.array_equal(orc.relu_f32(arr(g["input"])), arr(g["expected"]))
+    g = GOLD["relu_olt_f32_4x5"]
+    assert np.allclose(orc.relu_olt_f32(arr(g["input"])), arr(g["expected"]), rtol=1e-6)
+    # ugt and olt forms agree wherever the input is neither NaN nor -0.0
+    assert np.array_equal(orc.relu_f32(arr(g["input"])), orc.relu_olt_f32(arr(g["input"])))
+
+
+def test_relu_special_values(orc):
+    x = np.array([0x7fc00001, 0xffc12345, 0x80000000, 0x00000000, 0x00000001, 0x80000001, 0x7f800000, 0xff800000],
+                 np.uint32).view(np.float32)
+    y = orc.relu_f32(x).view(np.uint32)
+    # NaNs keep their payload, -0.0 -> +0.0, denormal+ kept, -inf -> 0
+    assert list(y) == [0x7fc00001, 0xffc12345, 0, 0, 1, 0, 0x7f800000, 0]
+    assert orc.relu_olt_f32(np.array([-0.0], np.float32)).view(np.uint32)[0] == 0x80000000
+
+
+def test_relu_bf16_golden(orc):
+    g = GOLD["relu_olt_bf16_4x5"]
+    x = orc.float_to_bfloat(arr(g["input"]))
+    y = orc.bfloat_to_float(orc.relu_16(x, "bf16"))
+    # the printed values are 2-3 digit roundings of bf16 numbers
+    assert np.allclose(y, arr(g["expected"]), rtol=4e-3)
+    assert np.array_equal(y == 0, arr(g["expected"]) == 0)
+
+
+# ---- silu ------------------------------------------------------------------------
+def test_silu_closed_forms(orc):
+    assert orc.silu_f32(np.array([0.0], np.float32))[0] == 0.0
+    x = np.linspace(-20, 20, 4001).astype(np.float32)
+    y = orc.silu_f32(x).astype(np.float64)
+    exact = x.astype(np.float64) / (1.0 + np.exp(-x.astype(np.float64)))
+    assert np.max(np.abs(y - exact) / np.maximum(np.abs(exact), 1e-30)) < 4e-7
+    # silu(x) - silu(-x) == x up to rounding
+    assert np.max(np.abs(y - y[::-1] - x)) < 4e-6
+    # limits: large positive -> x, large negative -> -0.0 / tiny
+    assert orc.silu_f32(np.array([100.0], np.float32))[0] == np.float32(100.0)
+    assert abs(float(orc.silu_f32(np.array([-100.0], np.float32))[0])) < 1e-40
+    # op order matters: the oracle multiplies sigmoid * x, with each step rounded
+    xv = np.float32(1.3)
+    e = np.float32(math.exp(-float(xv)))  # == expf for this input (checked below)
+    s = np.float32(1.0) / (e + np.float32(1.0))
+    assert orc.silu_f32(np.array([1.3], np.float32))[0] == np.float32(s * xv)
+
+
+def test_libm_expf_vs_correctly_rounded(orc):
+    """expf (host libm, what the reference's CPU lowering calls) is within 1 ulp
+    of the correctly rounded exponential everywhere sampled."""
+    x = orc.fill_uniform(200000, "f32", 99, -87.0, 88.0)
+    cr = np.exp(x.astype(np.float64)).astype(np.float32)
+    L = orc.lib()
+    import ctypes as C
+    got = np.array([L.oracle_expf_cr(C.c_float(float(v))) for v in x[:2000]], np.float32)
+    assert np.array_equal(got, cr[:2000])
+    e = orc.silu_f32  # noqa: F841 (silu uses expf; checked through ulp distance of exp itself)
+    libm = np.array([math.exp(float(v)) for v in x[:2000]])
+    assert np.max(orc.ulp_distance_f32(libm.astype(np.float32), cr[:2000])) <= 1
+
+
+# ---- softmax ---------------------------------------------------------------------
+@pytest.mark.parametrize("key", ["softmax_f32_10x20", "softmax_f32_10x20_spirv"])
+def test_softmax_golden(orc, key):
+    g = GOLD[key]
+    x = arr(g["input"], g["shape"])
+    want = arr(g["expected"], g["shape"])
+    for three_pass in (False, True):
+        got = orc.softmax_f32(x, three_pass)
+        assert np.max(np.abs(got - want) / want) < 2e-5  # six printed digits
+        assert orc.allclose_f32(got, want)
+
+
+def test_softmax_invariants(orc):
+    x = orc.fill_normal(64 * 1024, "f32", 5, 0.0, 2.0).reshape(64, 1024)
+    y = orc.softmax_f32(x)
+    assert np.max(np.abs(y.sum(axis=1, dtype=np.float64) - 1.0)) < 1e-5
+    # shift invariance by a power of two is exact when no rounding occurs in x + c
+    xi = np.round(x * 8) / 8
+    assert np.array_equal(orc.softmax_f32(xi), orc.softmax_f32((xi + 16).astype(np.float32)))
+    # an all-equal row of 1024 gives exactly 2^-10
+    eq = np.full((2, 1024), 3.3, np.float32)
+    assert np.all(orc.softmax_f32(eq) == np.float32(2.0 ** -10))
+    h = orc.softmax_16(orc.float_to_half(eq), "f16")
+    assert np.all(h == 0x1400)  # 2^-10 in f16
+    # against float64 evaluation
+    xd = x.astype(np.float64)
+    ed = np.exp(xd - xd.max(axis=1, keepdims=True))
+    assert np.max(np.abs(y - ed / ed.sum(axis=1, keepdims=True)) / y) < 2e-5
+
+
+# ---- reductions --------------------------------------------------------------------
+def test_sum_golden(orc):
+    g = GOLD["sum_f32_10x20"]
+    x = arr(g["input"], g["shape"])
+    assert orc.sum_all_f32(x) == g["expected"][0] == 2100.0
+    assert np.array_equal(orc.rowsum_f32(x), np.full(10, 210.0, np.float32))
+    assert np.array_equal(orc.reduce_outer_f32(x), np.arange(1, 21, dtype=np.float32) * 10)
+
+
+def test_wg_reduction_vectors(orc):
+    g = GOLD["wg_reduction_rows"]
+    x = np.repeat(np.arange(g["rows"], dtype=np.float32)[:, None], g["cols"], axis=1)
+    assert list(orc.rowsum_f32(x)) == g["expected"]
+    # reduction_2D_1D_cross_sg_intra_lane.mlir:105: sum of 0..31 down a column = 496
+    col = np.repeat(np.arange(32, dtype=np.float32)[:, None], 32, axis=1)
+    assert np.all(orc.reduce_outer_f32(col) == 496.0)
+    # reduction_3D_1D_*:91: 256*256 ones = 65536
+    assert orc.rowsum_f32(np.ones((1, 65536), np.float32))[0] == 65536.0
+
+
+def test_rowsum_is_sequential(orc):
+    # 2^24 + 1 + 1 ... stays at 2^24 when added left to right in f32
+    x = np.concatenate([[np.float32(2 ** 24)], np.ones(100, np.float32)])[None, :]
+    assert orc.rowsum_f32(x)[0] == np.float32(2 ** 24)
+    assert orc.rowsum_f32(x[:, ::-1].copy())[0] == np.float32(2 ** 24 + 100)
+    assert orc.rowsum_f32(np.ones((1, 3), np.float32), init=2.5)[0] == 5.5
+
+
+# ---- transpose ---------------------------------------------------------------------
+def test_transpose_golden(orc):
+    g = GOLD["transpose_f32_10x20"]
+    x = arr(g["input"], g["shape"])
+    assert np.array_equal(orc.transpose2d(x), arr(g["expected"], [20, 10]))
+    g = GOLD["transpose_bf16_10x20"]
+    xb = orc.float_to_bfloat(arr(g["input"], g["shape"]))
+    assert np.array_equal(orc.bfloat_to_float(orc.transpose2d(xb)), arr(g["expected"], [20, 10]))
+
+
+def test_transpose_closed_forms(orc):
+    x = np.arange(37 * 53, dtype=np.uint32).reshape(37, 53)
+    assert np.array_equal(orc.transpose2d(x), x.T)
+    assert np.array_equal(orc.transpose2d(orc.transpose2d(x)), x)
+    h = np.arange(17 * 9, dtype=np.uint16).reshape(17, 9)
+    assert np.array_equal(orc.transpose2d(h), h.T)
+    t = np.arange(5 * 7 * 3, dtype=np.uint32).reshape(5, 7, 3)
+    assert np.array_equal(orc.transpose3d(t), t.transpose(2, 1, 0))
+
+
+# ---- GEMM --------------------------------------------------------------------------
+def test_gemm_golden(orc):
+    g = GOLD["gemm_f32_3x3"]
+    c = orc.gemm(arr(g["A"], [3, 3]), arr(g["B"], [3, 3]), "f32", c=arr(g["C0"], [3, 3]))
+    assert np.allclose(c.ravel(), g["expected"], rtol=2e-6)
+    g = GOLD["gemm_f16_acc_f32_3x3"]
+    a, b = orc.float_to_half(arr(g["A"], [3, 3])), orc.float_to_half(arr(g["B"], [3, 3]))
+    c = orc.gemm(a, b, "f16", c=arr(g["C0"], [3, 3]))
+    assert np.max(np.abs(c.ravel() - arr(g["expected"]))) < 6e-5  # printed to 1e-4
+    assert orc.allclose_f32(c, arr(g["expected"], [3, 3]))
+    g = GOLD["gemm_bf16_acc_f32_3x3"]
+    a, b = orc.float_to_bfloat(arr(g["A"], [3, 3])), orc.float_to_bfloat(arr(g["B"], [3, 3]))
+    c = orc.gemm(a, b, "bf16", c=arr(g["C0"], [3, 3]))
+    assert np.max(np.abs(c.ravel() - arr(g["expected"]))) < 6e-5
+    g = GOLD["dot_f16_acc_f32_8x16x32"]
+    a = orc.float_to_half(np.full((g["M"], g["K"]), g["A_fill"], np.float32))
+    b = orc.float_to_half(np.full((g["K"], g["N"]), g["B_fill"], np.float32))
+    assert np.all(orc.gemm(a, b, "f16", out_round="f16") == g["expected_fill"])
+
+
+def test_gemm_closed_forms(orc):
+    # B = I  =>  C = A ; A[i,j] = j (gemm_4kx4kx4k_f16_f16_f32.mlir:109-138)
+    K = 96
+    a = orc.float_to_half(np.tile(np.arange(K, dtype=np.float32), (5, 1)))
+    eye = orc.float_to_half(np.eye(K, dtype=np.float32))
+    assert np.array_equal(orc.gemm(a, eye, "f16"), orc.half_to_float(a))
+    # small integers: exact, so it must equal the integer matmul whatever the order
+    ai = orc.fill_int(40 * 200, "bf16", 3, -4, 4).reshape(40, 200)
+    bi = orc.fill_int(200 * 24, "bf16", 4, -4, 4).reshape(200, 24)
+    want = orc.bfloat_to_float(ai).astype(np.int64) @ orc.bfloat_to_float(bi).astype(np.int64)
+    assert np.array_equal(orc.gemm(ai, bi, "bf16").astype(np.int64), want)
+    # the row-subset entry point is the same arithmetic
+    a = orc.fill_uniform(64 * 128, "f16", 7, -1, 1).reshape(64, 128)
+    b = orc.fill_uniform(128 * 32, "f16", 8, -1, 1).reshape(128, 32)
+    full = orc.gemm(a, b, "f16")
+    rows = np.array([0, 5, 63])
+    assert np.array_equal(orc.gemm_rows(a, b, rows, "f16"), full[rows])
+    # k-ascending f32 accumulation with a rounded product: compare with a literal loop
+    af, bf = orc.half_to_float(a), orc.half_to_float(b)
+    acc = np.float32(0)
+    for k in range(128):
+        acc = np.float32(acc + np.float32(af[3, k] * bf[k, 9]))
+    assert full[3, 9] == acc
+
+
+def test_bias_and_epilogue(orc):
+    c = np.arange(12, dtype=np.float32).reshape(3, 4)
+    bias = np.array([10, 20, 30, 40], np.float32)
+    assert np.array_equal(orc.bias_add_rows(c, bias), c + bias[None, :])
+    acc = orc.fill_normal(8 * 16, "f32", 11, 0, 3).reshape(8, 16)
+    b = orc.fill_normal(16, "f32", 12, 0, 0.1)
+    got = orc.bias_silu_bf16(acc, b)
+    want = orc.float_to_bfloat(orc.silu_f32((acc + b[None, :]).astype(np.float32)))
+    assert np.array_equal(got, want)
+
+
+# ---- allclose / max error -----------------------------------------------------------
+def test_allclose_formula(orc):
+    ref = np.array([1.0, 100.0, 0.0], np.float32)
+    assert orc.allclose_f32(ref + np.array([1e-3, 0.1, 9e-5], np.float32), ref)
+    assert not orc.allclose_f32(ref + np.array([1.2e-3, 0, 0], np.float32), ref)
+    assert not orc.allclose_f32(ref + np.array([0, 0, 1.1e-4], np.float32), ref)
+    # asymmetric in its arguments: the tolerance scales with the second one
+    assert orc.allclose_f32(np.array([0.0], np.float32), np.array([1e-4], np.float32))
+    ma, mr = orc.max_error_f32(np.array([1.0, 2.0], np.float32), np.array([1.5, 2.0], np.float32))
+    assert ma == 0.5 and abs(mr - 0.5 / 1.5) < 1e-12
+
+
+# ---- statistics -----------------------------------------------------------------------
+def test_stats_closed_forms(orc):
+    v = np.array([3, 1, 4, 1, 5, 9, 2, 6, 5, 3], np.float32)
+    assert orc.stat("min", v) == 1 and orc.stat("max", v) == 9
+    assert orc.stat("avg", v) == np.float32(3.9)
+    assert orc.stat("median_textbook", v) == 3.5
+    assert abs(orc.stat("variance", v) - float(np.var(v))) < 1e-5
+    assert abs(orc.stat("stddev", v) - float(np.std(v))) < 1e-5
+    s = np.sort(v)
+    assert orc.stat("p95", v) == s[9] and orc.stat("p5", v) == s[0]
+    assert orc.stat("middle_third_avg", v) == np.float32(s[3:7].sum() / 4)
+    assert orc.stat("median_reference", v) == (s[6] + s[5]) / 2  # pivot n/2+1: one past the middle
+
+
+def test_stats_match_reference_build(orc):
+    ref = orc.ref_stats()
+    if ref is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    import ctypes as C
+    rng = np.random.default_rng(5)
+    for n in (3, 4, 5, 10, 99, 100, 1000):
+        v = rng.random(n).astype(np.float32) * 3
+        p = C.c_void_p(v.ctypes.data)
+        pairs = [("min", "min"), ("max", "max"), ("avg", "avg"), ("median_reference", "median"),
+                 ("stddev", "stddev"), ("variance", "variance"), ("p95", "p95"), ("p5", "p5"),
+                 ("middle_third_avg", "middle_third_avg")]
+        for mine, theirs in pairs:
+            assert orc.stat(mine, v) == getattr(ref, "ref_stat_" + theirs)(p, n), (mine, n)
