@@ -29,7 +29,15 @@ constexpr int kThreads = 256;
 constexpr int kWavesPerBlock = kThreads / kWave;
 constexpr int64_t kWavePerRowMaxCols = 2048;
 
+template <bool kStream> __device__ __forceinline__ f32x4 loadf4(const f32x4 *p) {
+  if constexpr (kStream)
+    return __builtin_nontemporal_load(p);
+  else
+    return *p;
+}
+
 // Partial sum of one row over the lanes [tid, tid+stride, ...).
+template <bool kStream>
 __device__ __forceinline__ float row_partial(const float *__restrict__ row, int64_t cols, int tid, int stride) {
   float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
@@ -38,17 +46,17 @@ __device__ __forceinline__ float row_partial(const float *__restrict__ row, int6
     int64_t v = tid;
     // four independent 16-byte loads in flight per lane
     for (; v + 3 * int64_t(stride) < vecs; v += 4 * int64_t(stride)) {
-      f32x4 a = __builtin_nontemporal_load(src + v);
-      f32x4 b = __builtin_nontemporal_load(src + v + stride);
-      f32x4 c = __builtin_nontemporal_load(src + v + 2 * int64_t(stride));
-      f32x4 d = __builtin_nontemporal_load(src + v + 3 * int64_t(stride));
+      f32x4 a = loadf4<kStream>(src + v);
+      f32x4 b = loadf4<kStream>(src + v + stride);
+      f32x4 c = loadf4<kStream>(src + v + 2 * int64_t(stride));
+      f32x4 d = loadf4<kStream>(src + v + 3 * int64_t(stride));
       acc[0] += (a.x + a.y) + (a.z + a.w);
       acc[1] += (b.x + b.y) + (b.z + b.w);
       acc[2] += (c.x + c.y) + (c.z + c.w);
       acc[3] += (d.x + d.y) + (d.z + d.w);
     }
     for (; v < vecs; v += stride) {
-      f32x4 a = __builtin_nontemporal_load(src + v);
+      f32x4 a = loadf4<kStream>(src + v);
       acc[0] += (a.x + a.y) + (a.z + a.w);
     }
     for (int64_t c = vecs * 4 + tid; c < cols; c += stride)
@@ -66,12 +74,16 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_rowsum_f32(const flo
                                                                       int64_t cols, float init) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
+  // the input is read exactly once: stream it past the caches (non-temporal)
+  constexpr bool stream = true;
   if (cols > kWavePerRowMaxCols) {
     __shared__ float partial[kWavesPerBlock];
     const int64_t row = blockIdx.x;
     if (row >= rows)
       return;
-    float s = wave_sum(row_partial(in + row * cols, cols, threadIdx.x, kThreads));
+    const float p = stream ? row_partial<true>(in + row * cols, cols, threadIdx.x, kThreads)
+                           : row_partial<false>(in + row * cols, cols, threadIdx.x, kThreads);
+    float s = wave_sum(p);
     if (lane == 0)
       partial[wave] = s;
     __syncthreads();
@@ -81,7 +93,9 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_rowsum_f32(const flo
     const int64_t row = int64_t(blockIdx.x) * kWavesPerBlock + wave;
     if (row >= rows)
       return;
-    float s = wave_sum(row_partial(in + row * cols, cols, lane, kWave));
+    const float p = stream ? row_partial<true>(in + row * cols, cols, lane, kWave)
+                           : row_partial<false>(in + row * cols, cols, lane, kWave);
+    float s = wave_sum(p);
     if (lane == 0)
       out[row] = init + s;
   }

@@ -5,17 +5,23 @@
 // temporaries; single-kernel streaming form in
 // test/Integration/Dialect/XeGPU/WG/softmax_intra_sg_cross_lane.mlir:118-205.
 //
-// Here: ONE kernel, input read once and output written once.  A wavefront owns
-// a row and keeps it in registers (128-bit loads, 8 x 16-bit or 4 x f32 per
-// load), max and sum are wavefront-64 butterfly reductions, internals are f32.
-// Rows too long for registers, or whose length breaks 16-byte alignment, go
-// through a workgroup-per-row path that re-reads the row from cache.
-//
-// 16-bit I/O follows the reference's policy for 16-bit types on the GPU:
-// extend to f32, compute, truncate (docs/Transforms/BF16ToGpu.md:17-26).
+// Here: ONE kernel, input read once from HBM and output written once.
+//  * rows of up to 128 lanes x 16 B (1024 16-bit / 512 f32 elements): a
+//    wavefront owns TWO rows at a time and keeps them in registers; max and sum
+//    are wavefront-64 butterfly reductions.  Two rows per wavefront and a
+//    64-register budget (8 wavefronts per SIMD) keep enough loads in flight to
+//    cover HBM latency.
+//  * rows of up to 4096 elements: a workgroup owns a row and stages it in LDS
+//    as f32 (read once, three passes over LDS).
+//  * longer rows, or bases that break 16-byte alignment on the register path:
+//    workgroup per row, re-reading the row from cache.
+// Internals are f32; 16-bit I/O follows the reference's policy for 16-bit types
+// on the GPU: extend to f32, compute, truncate (docs/Transforms/BF16ToGpu.md:17-26).
 //
 // Arguments: (in, out, rows: i64, cols: i64).
-// Launch: block (256,1,1); grid (ceil(rows / 4), 1, 1)  [4 wavefronts = 4 rows].
+// Launch: block (256,1,1); any grid >= 1 is correct (workgroups stride over the
+// rows); the catalogue sizes it to one pass: ceil(rows/8) for register-resident
+// rows, else min(rows, 65535 * 16).
 
 #include "device_common.h"
 
@@ -24,9 +30,10 @@ using namespace imexhip;
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kRowsPerBlock = kThreads / kWave;
-// Up to kMaxChunks 16-byte chunks per lane live in registers.
-constexpr int kMaxChunks = 8;
+constexpr int kWaves = kThreads / kWave;
+constexpr int kRegChunks = 2;          // 16-byte chunks per lane and row on the register path
+constexpr int kRowsPerWave = 2;
+constexpr int kLdsCols = 4096;         // longest row staged in LDS
 
 enum class Dt { F32, F16, BF16 };
 
@@ -102,58 +109,78 @@ __device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
 // (softmax_gpu.mlir.in:6).
 constexpr float kMaxInit = -3.40282347e+38f;
 
-// ---- wavefront-per-row, row resident in registers ---------------------------
-template <Dt D, int kChunks>
-__device__ __forceinline__ void softmax_row_in_regs(const void *in, void *out, int64_t row, int64_t cols) {
+// ---- register path: a wavefront owns kRowsPerWave rows ---------------------------
+template <Dt D, bool kStream>
+__device__ __forceinline__ void softmax_rows_in_regs(const void *in, void *out, int64_t rows, int64_t cols) {
   using E = Elem<D>;
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t vecsPerRow = cols / E::kPerVec; // cols is a multiple of kPerVec here
-  const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(in) + row * cols * E::kBytes);
-  u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + row * cols * E::kBytes);
-
-  float x[kChunks][E::kPerVec];
-  float m = kMaxInit;
+  const int wave = threadIdx.x / kWave;
+  const int64_t vecsPerRow = cols / E::kPerVec;
+  const int64_t rowBytes = cols * E::kBytes;
+  const int64_t groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
+  for (int64_t g = int64_t(blockIdx.x) * kWaves + wave; g < groups; g += int64_t(gridDim.x) * kWaves) {
+    float x[kRowsPerWave][kRegChunks][E::kPerVec];
+    u32x4 raw[kRowsPerWave][kRegChunks];
+    // all loads of both rows first
 #pragma unroll
-  for (int c = 0; c < kChunks; ++c) {
-    const int64_t v = int64_t(c) * kWave + lane;
-    if (v < vecsPerRow) {
-      E::unpack(__builtin_nontemporal_load(src + v), x[c]);
+    for (int r = 0; r < kRowsPerWave; ++r) {
+      const int64_t row = g * kRowsPerWave + r;
+      const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(in) + row * rowBytes);
 #pragma unroll
-      for (int i = 0; i < E::kPerVec; ++i)
-        m = fmaxf(m, x[c][i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < E::kPerVec; ++i)
-        x[c][i] = kMaxInit;
+      for (int c = 0; c < kRegChunks; ++c) {
+        const int64_t v = int64_t(c) * kWave + lane;
+        if (row < rows && v < vecsPerRow)
+          raw[r][c] = load128<kStream>(src + v);
+      }
     }
-  }
-  m = wave_max(m);
-
-  float s = 0.0f;
 #pragma unroll
-  for (int c = 0; c < kChunks; ++c) {
-    const bool live = int64_t(c) * kWave + lane < vecsPerRow;
+    for (int r = 0; r < kRowsPerWave; ++r) {
+      const int64_t row = g * kRowsPerWave + r;
+      if (row >= rows)
+        continue; // uniform across the wavefront
+      float m = kMaxInit;
 #pragma unroll
-    for (int i = 0; i < E::kPerVec; ++i) {
-      x[c][i] = live ? fast_exp(x[c][i] - m) : 0.0f;
-      s += x[c][i];
-    }
-  }
-  s = wave_sum(s);
-
+      for (int c = 0; c < kRegChunks; ++c) {
+        const bool live = int64_t(c) * kWave + lane < vecsPerRow;
+        if (live)
+          E::unpack(raw[r][c], x[r][c]);
 #pragma unroll
-  for (int c = 0; c < kChunks; ++c) {
-    const int64_t v = int64_t(c) * kWave + lane;
-    if (v < vecsPerRow) {
+        for (int i = 0; i < E::kPerVec; ++i) {
+          x[r][c][i] = live ? x[r][c][i] : kMaxInit;
+          m = fmaxf(m, x[r][c][i]);
+        }
+      }
+      m = wave_max(m);
+      float s = 0.0f;
 #pragma unroll
-      for (int i = 0; i < E::kPerVec; ++i)
-        x[c][i] = x[c][i] / s;
-      __builtin_nontemporal_store(E::pack(x[c]), dst + v);
+      for (int c = 0; c < kRegChunks; ++c) {
+        const bool live = int64_t(c) * kWave + lane < vecsPerRow;
+#pragma unroll
+        for (int i = 0; i < E::kPerVec; ++i) {
+          x[r][c][i] = live ? fast_exp(x[r][c][i] - m) : 0.0f;
+          s += x[r][c][i];
+        }
+      }
+      s = wave_sum(s);
+      // one IEEE division per row, then multiplies (differs from z / s by at
+      // most an f32 rounding, far inside the 1e-3 bar)
+      const float inv = 1.0f / s;
+      u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + row * rowBytes);
+#pragma unroll
+      for (int c = 0; c < kRegChunks; ++c) {
+        const int64_t v = int64_t(c) * kWave + lane;
+        if (v < vecsPerRow) {
+#pragma unroll
+          for (int i = 0; i < E::kPerVec; ++i)
+            x[r][c][i] = x[r][c][i] * inv;
+          store128<kStream>(E::pack(x[r][c]), dst + v);
+        }
+      }
     }
   }
 }
 
-// ---- workgroup-per-row, any length and alignment ------------------------------
+// ---- workgroup reductions -------------------------------------------------------------
 __device__ __forceinline__ float block_reduce(float v, bool isMax, float *scratch) {
   v = isMax ? wave_max(v) : wave_sum(v);
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
@@ -163,11 +190,75 @@ __device__ __forceinline__ float block_reduce(float v, bool isMax, float *scratc
   __syncthreads();
   float r = scratch[0];
 #pragma unroll
-  for (int w = 1; w < kRowsPerBlock; ++w)
+  for (int w = 1; w < kWaves; ++w)
     r = isMax ? fmaxf(r, scratch[w]) : r + scratch[w];
   return r;
 }
 
+// ---- LDS path: a workgroup owns a row, staged once in LDS as f32 ------------------------
+template <Dt D>
+__device__ __forceinline__ void softmax_row_in_lds(const void *in, void *out, int64_t row, int64_t cols,
+                                                   float *rowBuf, float *scratch, bool vec) {
+  using E = Elem<D>;
+  const int64_t base = row * cols;
+  float m = kMaxInit;
+  // Vector path: element i of 16-byte vector v lives at rowBuf[i * vecs + v], so
+  // neighbouring lanes touch neighbouring LDS words (no bank conflicts).
+  const int64_t vecs = cols / E::kPerVec;
+  if (vec) {
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(in) + base * E::kBytes);
+    for (int64_t v = threadIdx.x; v < vecs; v += kThreads) {
+      float f[E::kPerVec];
+      E::unpack(src[v], f);
+#pragma unroll
+      for (int i = 0; i < E::kPerVec; ++i) {
+        rowBuf[i * vecs + v] = f[i];
+        m = fmaxf(m, f[i]);
+      }
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < cols; c += kThreads) {
+      const float f = E::load(in, base + c);
+      rowBuf[c] = f;
+      m = fmaxf(m, f);
+    }
+  }
+  m = block_reduce(m, true, scratch); // its barriers also publish rowBuf
+  float s = 0.0f;
+  // each thread revisits exactly the elements it wrote: no barrier needed until the sum
+  if (vec) {
+    for (int64_t v = threadIdx.x; v < vecs; v += kThreads)
+#pragma unroll
+      for (int i = 0; i < E::kPerVec; ++i) {
+        const float e = fast_exp(rowBuf[i * vecs + v] - m);
+        rowBuf[i * vecs + v] = e;
+        s += e;
+      }
+  } else {
+    for (int64_t c = threadIdx.x; c < cols; c += kThreads) {
+      const float e = fast_exp(rowBuf[c] - m);
+      rowBuf[c] = e;
+      s += e;
+    }
+  }
+  s = block_reduce(s, false, scratch);
+  if (vec) {
+    u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + base * E::kBytes);
+    for (int64_t v = threadIdx.x; v < vecs; v += kThreads) {
+      float f[E::kPerVec];
+#pragma unroll
+      for (int i = 0; i < E::kPerVec; ++i)
+        f[i] = rowBuf[i * vecs + v] / s;
+      dst[v] = E::pack(f);
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < cols; c += kThreads)
+      E::store(out, base + c, rowBuf[c] / s);
+  }
+  __syncthreads(); // rowBuf is reused by the next row
+}
+
+// ---- any length: workgroup per row, three passes over the (cached) input ----------------
 template <Dt D>
 __device__ __forceinline__ void softmax_row_streamed(const void *in, void *out, int64_t row, int64_t cols,
                                                      float *scratch) {
@@ -188,46 +279,36 @@ __device__ __forceinline__ void softmax_row_streamed(const void *in, void *out, 
 template <Dt D>
 __device__ __forceinline__ void softmax_kernel(const void *in, void *out, int64_t rows, int64_t cols) {
   using E = Elem<D>;
-  __shared__ float scratch[kRowsPerBlock];
+  __shared__ float scratch[kWaves];
+  __shared__ __attribute__((aligned(16))) float rowBuf[kLdsCols];
   const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
                        (cols % E::kPerVec) == 0;
-  const int64_t chunks = (cols / E::kPerVec + kWave - 1) / kWave;
-  const int64_t row0 = int64_t(blockIdx.x) * kRowsPerBlock;
-  if (aligned && chunks <= kMaxChunks) {
-    const int64_t row = row0 + threadIdx.x / kWave;
-    if (row >= rows)
-      return;
-    if (chunks <= 1)
-      softmax_row_in_regs<D, 1>(in, out, row, cols);
-    else if (chunks <= 2)
-      softmax_row_in_regs<D, 2>(in, out, row, cols);
-    else if (chunks <= 4)
-      softmax_row_in_regs<D, 4>(in, out, row, cols);
-    else
-      softmax_row_in_regs<D, kMaxChunks>(in, out, row, cols);
+  if (aligned && cols <= int64_t(kRegChunks) * kWave * E::kPerVec) {
+    softmax_rows_in_regs<D, true>(in, out, rows, cols); // non-temporal: measured faster hot and cold
+  } else if (cols <= kLdsCols) {
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x)
+      softmax_row_in_lds<D>(in, out, row, cols, rowBuf, scratch, aligned);
   } else {
-    // Uniform per workgroup: every thread walks the same rows, so the barriers
-    // inside block_reduce are reached by all of them.
-    for (int r = 0; r < kRowsPerBlock; ++r) {
-      const int64_t row = row0 + r;
-      if (row >= rows)
-        break;
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x)
       softmax_row_streamed<D>(in, out, row, cols, scratch);
-    }
   }
 }
 
 } // namespace
 
-extern "C" __global__ __launch_bounds__(kThreads) void imex_softmax_f32(const float *in, float *out,
-                                                                       int64_t rows, int64_t cols) {
+// 8 wavefronts per SIMD (64 registers per lane) so two rows per wavefront still
+// leave room for full occupancy.
+#define IMEX_SOFTMAX_BOUNDS __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8)))
+
+extern "C" __global__ IMEX_SOFTMAX_BOUNDS void imex_softmax_f32(const float *in, float *out, int64_t rows,
+                                                                int64_t cols) {
   softmax_kernel<Dt::F32>(in, out, rows, cols);
 }
-extern "C" __global__ __launch_bounds__(kThreads) void imex_softmax_f16(const uint16_t *in, uint16_t *out,
-                                                                       int64_t rows, int64_t cols) {
+extern "C" __global__ IMEX_SOFTMAX_BOUNDS void imex_softmax_f16(const uint16_t *in, uint16_t *out, int64_t rows,
+                                                                int64_t cols) {
   softmax_kernel<Dt::F16>(in, out, rows, cols);
 }
-extern "C" __global__ __launch_bounds__(kThreads) void imex_softmax_bf16(const uint16_t *in, uint16_t *out,
-                                                                        int64_t rows, int64_t cols) {
+extern "C" __global__ IMEX_SOFTMAX_BOUNDS void imex_softmax_bf16(const uint16_t *in, uint16_t *out, int64_t rows,
+                                                                 int64_t cols) {
   softmax_kernel<Dt::BF16>(in, out, rows, cols);
 }

@@ -25,7 +25,7 @@ extern const unsigned char imex_blob_gemm[], imex_blob_gemm_end[];
 namespace {
 
 enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm };
-enum class Shape { Eltwise32, Eltwise16, SoftmaxRows, RowSum, ReduceOuter, Transpose2D, Transpose3D, Gemm, GemmFixed4k };
+enum class Shape { Eltwise32, Eltwise16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmFixed4k };
 
 struct Entry {
   const char *name;
@@ -40,18 +40,18 @@ const Entry kEntries[] = {
     {"imex_relu_f16", "(in: f16*, out: f16*, n: i64)", Module::Eltwise, Shape::Eltwise16, 1},
     {"imex_relu_bf16", "(in: bf16*, out: bf16*, n: i64)", Module::Eltwise, Shape::Eltwise16, 1},
     {"imex_silu_f32", "(in: f32*, out: f32*, n: i64)", Module::Eltwise, Shape::Eltwise32, 1},
-    {"imex_softmax_f32", "(in: f32*, out: f32*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows, 2},
-    {"imex_softmax_f16", "(in: f16*, out: f16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows, 2},
-    {"imex_softmax_bf16", "(in: bf16*, out: bf16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows, 2},
+    {"imex_softmax_f32", "(in: f32*, out: f32*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows32, 2},
+    {"imex_softmax_f16", "(in: f16*, out: f16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows16, 2},
+    {"imex_softmax_bf16", "(in: bf16*, out: bf16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows16, 2},
     {"imex_rowsum_f32", "(in: f32*, out: f32*, rows: i64, cols: i64, init: f32)", Module::Reduce, Shape::RowSum, 2},
     {"imex_reduce_outer_f32", "(in: f32*, out: f32*, outer: i64, inner: i64, init: f32)", Module::Reduce,
      Shape::ReduceOuter, 2},
-    {"imex_transpose2d_b32", "(in: b32*, out: b32*, rows: i64, cols: i64)", Module::Transpose, Shape::Transpose2D, 2},
-    {"imex_transpose2d_b16", "(in: b16*, out: b16*, rows: i64, cols: i64)", Module::Transpose, Shape::Transpose2D, 2},
+    {"imex_transpose2d_b32", "(in: b32*, out: b32*, rows: i64, cols: i64)", Module::Transpose, Shape::Transpose2D32, 2},
+    {"imex_transpose2d_b16", "(in: b16*, out: b16*, rows: i64, cols: i64)", Module::Transpose, Shape::Transpose2D16, 2},
     {"imex_transpose3d_b32", "(in: b32*, out: b32*, d0: i64, d1: i64, d2: i64)", Module::Transpose,
-     Shape::Transpose3D, 3},
+     Shape::Transpose3D32, 3},
     {"imex_transpose3d_b16", "(in: b16*, out: b16*, d0: i64, d1: i64, d2: i64)", Module::Transpose,
-     Shape::Transpose3D, 3},
+     Shape::Transpose3D16, 3},
     {"imex_gemm_f16_f16_f32", "(A: f16*, B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
     {"imex_gemm_f16_f16_f32_acc", "(A: f16*, B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
     {"imex_gemm_bf16_bf16_f32", "(A: bf16*, B: bf16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
@@ -128,26 +128,38 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
   case Shape::Eltwise16: // 256 lanes x 4 vectors x 8 elements
     grid[0] = ceilDiv(dims[0], 8192);
     break;
-  case Shape::SoftmaxRows: // one wavefront per row, four per workgroup
-    grid[0] = ceilDiv(dims[0], 4);
+  case Shape::SoftmaxRows32:
+  case Shape::SoftmaxRows16: {
+    // Rows of up to 128 x 16 B stay in registers, two per wavefront (eight per
+    // workgroup); longer rows take a workgroup each.  The kernel strides over
+    // the rows, so any grid is correct; this one covers them in a single pass.
+    const int64_t regCols = e->shape == Shape::SoftmaxRows16 ? 1024 : 512;
+    grid[0] = dims[1] <= regCols ? ceilDiv(dims[0], 8) : static_cast<size_t>(dims[0] < 1048560 ? dims[0] : 1048560);
     if (dims[1] == 0)
       grid[0] = 0;
     break;
+  }
   case Shape::RowSum: // workgroup per row above 2048 columns, else wavefront per row
     grid[0] = dims[1] > 2048 ? static_cast<size_t>(dims[0]) : ceilDiv(dims[0], 4);
     break;
   case Shape::ReduceOuter: // four outputs per lane
     grid[0] = ceilDiv(dims[1], 1024);
     break;
-  case Shape::Transpose2D:
-    grid[0] = ceilDiv(dims[1], 64);
-    grid[1] = ceilDiv(dims[0], 64);
+  case Shape::Transpose2D32: // 64 x 64 tiles
+  case Shape::Transpose2D16: { // 128 x 128 tiles
+    const int64_t tile = e->shape == Shape::Transpose2D32 ? 64 : 128;
+    grid[0] = ceilDiv(dims[1], tile);
+    grid[1] = ceilDiv(dims[0], tile);
     break;
-  case Shape::Transpose3D:
-    grid[0] = ceilDiv(dims[2], 64);
-    grid[1] = ceilDiv(dims[0], 64);
+  }
+  case Shape::Transpose3D32:
+  case Shape::Transpose3D16: {
+    const int64_t tile = e->shape == Shape::Transpose3D32 ? 64 : 128;
+    grid[0] = ceilDiv(dims[2], tile);
+    grid[1] = ceilDiv(dims[0], tile);
     grid[2] = static_cast<size_t>(dims[1]);
     break;
+  }
   case Shape::Gemm: {
     const int64_t M = dims[0], N = dims[1], K = dims[2];
     const bool tileable = M > 0 && N > 0 && K > 0 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0;

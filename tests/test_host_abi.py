@@ -63,11 +63,13 @@ def test_launch_shapes(host):
     assert ls("imex_relu_f32", [1])[0] == (1, 1, 1)
     assert ls("imex_relu_f32", [0])[0][0] == 0  # nothing to launch
     assert ls("imex_relu_bf16", [8193])[0] == (2, 1, 1)
-    assert ls("imex_softmax_f16", [16384, 1024])[0] == (4096, 1, 1)
+    assert ls("imex_softmax_f16", [16384, 1024])[0] == (2048, 1, 1)
+    assert ls("imex_softmax_f32", [16, 2000])[0] == (16, 1, 1)
     assert ls("imex_rowsum_f32", [8192, 8192])[0] == (8192, 1, 1)
     assert ls("imex_rowsum_f32", [8, 256])[0] == (2, 1, 1)
     assert ls("imex_reduce_outer_f32", [32, 16 * 512 * 512])[0] == (4096, 1, 1)
-    assert ls("imex_transpose2d_b16", [8192, 8192])[0] == (128, 128, 1)
+    assert ls("imex_transpose2d_b16", [8192, 8192])[0] == (64, 64, 1)
+    assert ls("imex_transpose2d_b32", [4096, 4096])[0] == (64, 64, 1)
     assert ls("imex_transpose2d_b32", [10, 20])[0] == (1, 1, 1)
     assert ls("imex_transpose3d_b32", [16, 96, 96])[0] == (2, 1, 96)
     assert ls("imex_gemm_f16_f16_f32", [4096, 4096, 4096])[0] == (256, 1, 1)
