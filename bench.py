@@ -226,7 +226,7 @@ def main():
         "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic (seeded std::mt19937 stream, inputs resident in HBM)",
         "config": {"workload": "BASELINE configs[3]: " + head.describe, "kernel": head.kernel,
-                   "launch": "grid (256,1,1) x block (256,1,1)", "device": info["name"],
+                   "launch": "grid (256,1,1) x block (512,1,1)", "device": info["name"],
                    "cus": info["cus"], "clock_mhz": info["clock_khz"] / 1e3},
         "roofline": dict(roofline(head, kernel_ms), event_ms_per_step=round(event_ms, 5),
                          kernel_ms=round(kernel_ms, 5)),

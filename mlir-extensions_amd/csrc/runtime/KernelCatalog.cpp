@@ -160,14 +160,17 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     grid[2] = static_cast<size_t>(dims[1]);
     break;
   }
-  case Shape::Gemm: {
+  case Shape::Gemm: { // 512 lanes: eight wavefronts per 256 x 256 tile
     const int64_t M = dims[0], N = dims[1], K = dims[2];
     const bool tileable = M > 0 && N > 0 && K > 0 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0;
-    grid[0] = tileable ? static_cast<size_t>((M / 256) * (N / 256)) : ceilDiv(M * N, 256);
+    block[0] = 512;
+    grid[0] = tileable ? static_cast<size_t>((M / 256) * (N / 256)) : ceilDiv(M * N, 512);
     break;
   }
-  case Shape::GemmFixed4k:
-    grid[0] = 256;
+  case Shape::GemmFixed4k: // the reference's own launch: blocks (16,16,1), threads (512,1,1)
+    block[0] = 512;
+    grid[0] = 16;
+    grid[1] = 16;
     break;
   }
   // A grid component of 0 means there is nothing to launch.

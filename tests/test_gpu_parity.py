@@ -297,7 +297,7 @@ def test_gemm_config_f16_4096(host, orc, stream):
     fn = stream.kernel("imex_gemm_4kx4kx4k_f16_f16_f32")
     descs, keep = host._pack_params([d_a, d_b, d_c])
     import ctypes as C
-    stream.rt.gpuLaunchKernel(stream.handle, fn, 16, 16, 1, 256, 1, 1, 0, C.cast(descs, C.c_void_p), None)
+    stream.rt.gpuLaunchKernel(stream.handle, fn, 16, 16, 1, 512, 1, 1, 0, C.cast(descs, C.c_void_p), None)
     stream.wait()
     fixed = stream.from_device(d_c, (M, N), np.float32)
     for p in (d_a, d_b, d_c):

@@ -72,10 +72,10 @@ def test_launch_shapes(host):
     assert ls("imex_transpose2d_b32", [4096, 4096])[0] == (64, 64, 1)
     assert ls("imex_transpose2d_b32", [10, 20])[0] == (1, 1, 1)
     assert ls("imex_transpose3d_b32", [16, 96, 96])[0] == (2, 1, 96)
-    assert ls("imex_gemm_f16_f16_f32", [4096, 4096, 4096])[0] == (256, 1, 1)
+    assert ls("imex_gemm_f16_f16_f32", [4096, 4096, 4096]) == ((256, 1, 1), (512, 1, 1), 0)
     assert ls("imex_gemm_bf16_bias_silu_bf16", [4096, 11008, 4096])[0] == (16 * 43, 1, 1)
     assert ls("imex_gemm_f16_f16_f32", [3, 3, 3])[0] == (1, 1, 1)
-    assert ls("imex_gemm_4kx4kx4k_f16_f16_f32", [])[0] == (256, 1, 1)
+    assert ls("imex_gemm_4kx4kx4k_f16_f16_f32", []) == ((16, 16, 1), (512, 1, 1), 0)
     with pytest.raises(ValueError):
         ls("imex_relu_f32", [1, 2])
     with pytest.raises(ValueError):
