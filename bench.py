@@ -72,7 +72,7 @@ def build_workloads(host, orc, stream, only):
         a = orc.fill_uniform(M * K, "f16", 20246, -1.0, 1.0).reshape(M, K)
         b = orc.fill_uniform(K * N, "f16", 20247, -1.0, 1.0).reshape(K, N)
         cur.args = [dev(a), dev(b), out(M * N * 4), M, N, K]
-        rows = 256
+        rows = 2048
 
         def cpu(a=a, b=b, rows=rows):
             ms = orc.time_gemm_rows(a, b, rows, "f16")
@@ -152,13 +152,33 @@ def build_workloads(host, orc, stream, only):
     return wl
 
 
+def measured_traffic():
+    """HBM-side bytes per launch from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE
+    summary (profiles/hbm_traffic_fetch_write_pmc.txt); {} if it is absent."""
+    path = os.path.join(REPO, "profiles", "hbm_traffic_fetch_write_pmc.txt")
+    out = {}
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if line.startswith("#") or len(parts) != 8:
+                    continue
+                out[parts[0]] = int(parts[7])
+    except OSError:
+        pass
+    return out
+
+
+TRAFFIC = measured_traffic()
+
+
 def roofline(w, ms):
     if w.bound == "mfma":
         achieved, peak, unit = w.work / (ms * 1e9), MFMA_PEAK_TFLOPS, "TFLOP/s"
     else:
         achieved, peak, unit = w.work / (ms * 1e6), HBM_PEAK_GBS, "GB/s"
     return {"bound": w.bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 4), "traffic": None}
+            "frac": round(achieved / peak, 4), "traffic": TRAFFIC.get(w.name)}
 
 
 def measure_secondary(stream, w, rounds):
@@ -200,21 +220,31 @@ def main():
     workloads = build_workloads(host, orc, stream, only)
     log("inputs generated and resident in HBM after %.1f s" % (time.time() - t_setup))
 
+    # Host -> device copy rate through gpuMemCopy (pageable host memory), for the
+    # PCIe-inclusive figure quoted in the design notes; never part of `value`.
+    probe = np.zeros(64 << 20, np.uint8)
+    d_probe = stream.alloc(probe.nbytes)
+    stream.copy(d_probe, probe.ctypes.data, probe.nbytes)
+    t = time.perf_counter()
+    stream.copy(d_probe, probe.ctypes.data, probe.nbytes)
+    h2d_gbs = probe.nbytes / (time.perf_counter() - t) / 1e9
+    stream.free(d_probe)
+    log("gpuMemCopy host->device: %.1f GB/s" % h2d_gbs)
+
     head = workloads[0]
     K, W = args.steps, args.warmup
-    ev0 = None
+    step = stream.prepare(head.kernel, head.dims, head.args)
     for _ in range(max(W, 1)):
-        ev0 = stream.launch(head.kernel, head.dims, head.args)
+        step()
     stream.wait()
     t0 = time.perf_counter()
-    ev1 = None
+    ev0 = stream.timestamp()  # HIP events on the launch stream bracket exactly the K timed launches
     for _ in range(K):
-        ev1 = stream.launch(head.kernel, head.dims, head.args)
+        step()
+    ev1 = stream.timestamp()
     stream.wait()
     t1 = time.perf_counter()
     wall_ms = (t1 - t0) * 1e3 / K
-    # ev0 was recorded before the timed launches were enqueued (and the stream
-    # was idle at t0), so ev0 -> ev1 spans exactly the K timed launches.
     event_ms = stream.elapsed_ms(ev0, ev1) / K
     # device-side duration of a launch: back-to-back launches from C, no Python in the loop
     kernel_ms = stream.profile(head.kernel, head.dims, head.args, warmups=3, rounds=K, mode=1)[0] / K
@@ -227,7 +257,8 @@ def main():
         "dtype": "f16", "data": "synthetic (seeded std::mt19937 stream, inputs resident in HBM)",
         "config": {"workload": "BASELINE configs[3]: " + head.describe, "kernel": head.kernel,
                    "launch": "grid (256,1,1) x block (512,1,1)", "device": info["name"],
-                   "cus": info["cus"], "clock_mhz": info["clock_khz"] / 1e3},
+                   "cus": info["cus"], "clock_mhz": info["clock_khz"] / 1e3,
+                   "gpuMemCopy_h2d_GBps": round(h2d_gbs, 1)},
         "roofline": dict(roofline(head, kernel_ms), event_ms_per_step=round(event_ms, 5),
                          kernel_ms=round(kernel_ms, 5)),
     }

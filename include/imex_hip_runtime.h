@@ -82,7 +82,8 @@ void *gpuKernelGet(void *queue, void *module, const char *name);
  * workgroups.  If sharedMemBytes != 0 the last ParamDesc is the placeholder
  * for dynamic shared memory and is not passed as an argument.  Only the low 32
  * bits of sharedMemBytes are used (the call site passes i32).  Returns an
- * event recorded after the launch, owned by the stream.
+ * event that stands for "after this launch" on the stream, owned by the
+ * stream; it can be listed in a later launch's depEvents (on any stream).
  * Environment (LevelZeroRuntimeWrappers.cpp:521-597): IMEX_ENABLE_PROFILING,
  * IMEX_PROFILING_RUNS (default 1000), IMEX_PROFILING_WARMUPS (default 3),
  * IMEX_ENABLE_CACHE_FLUSHING, plus IMEX_CACHE_FLUSH_BYTES (default 512 MiB). */
@@ -129,7 +130,12 @@ int imexHipProfileKernel(void *queue, void *kernel, size_t gridX, size_t gridY, 
                          void *params, int warmups, int rounds, size_t flushBytes, int mode,
                          float *times_ms);
 
-/* Milliseconds between two events returned by gpuLaunchKernel on one stream. */
+/* Records a timestamp event at the stream's current tail (owned by the stream). */
+void *imexHipRecordTimestamp(void *queue);
+
+/* Milliseconds between two events of one stream.  Use imexHipRecordTimestamp
+ * events for timing: an event returned by gpuLaunchKernel is an ordering point,
+ * whose timestamp is taken when it is first used. */
 float imexHipEventElapsedMs(void *startEvent, void *stopEvent);
 
 /* out[9] = avg, min, max, median, stddev, variance, P95, P5, middle-third avg

@@ -1,0 +1,233 @@
+//===- imex_hip_bench.cpp - C++ host driver over the gpu* runtime ABI ------===//
+//
+// Does, in plain C++ through the C ABI only, what IMEX's JIT'd `main` plus the
+// `bench_imex` script do for one benchmark workload
+// (benchmarks/bench_imex.in:23-92, lib/Conversion/GPUXToLLVM/GPUXToLLVMPass.cpp:
+// 373-383,508-518,691-710):
+//
+//   gpuCreateStream -> gpuMemAlloc -> fill on the host -> gpuMemCopy (H2D) ->
+//   gpuModuleLoad + gpuKernelGet + gpuLaunchKernel(ParamDesc[]) -> gpuWait ->
+//   gpuMemCopy (D2H) -> gpuMemFree -> gpuStreamDestroy
+//
+// and prints one "<workload>: the kernel execution time is (ms, on HIP
+// runtime):avg: ..." line per workload, the line bench_imex greps into
+// report.txt (bench_imex.in:87-91).
+//
+//   imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--launch-only N] <workload>...
+//   imex-hip-bench --list
+//
+//   -l             accepted for bench_imex compatibility (the HIP runtime is the only backend here)
+//   --launch-only  skip the timing loop and just launch the kernel N times (for
+//                  rocprofv3 counter runs, which time and count every dispatch themselves)
+//
+//===----------------------------------------------------------------------===//
+
+#include "imex_hip_kernels.h"
+#include "imex_hip_runtime.h"
+#include "imex_runner_utils.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+namespace {
+
+enum class Elem { F32, F16, BF16 };
+size_t elemBytes(Elem e) { return e == Elem::F32 ? 4 : 2; }
+
+struct Tensor {
+  Elem elem;
+  std::vector<int64_t> shape;
+  bool isInput;
+  float lo, hi; // uniform fill range for inputs
+};
+
+struct Workload {
+  const char *name;
+  const char *kernel;
+  std::vector<int64_t> dims;    // what imexHipKernelLaunchShape takes
+  std::vector<Tensor> tensors;  // kernel pointer arguments, in order
+  std::vector<int64_t> indexArgs; // i64 arguments after the pointers
+  bool hasInit;                 // trailing f32 `init` argument (reductions)
+  double work;                  // algorithmic bytes or flops per launch
+  bool mfma;                    // roofline: MFMA (TFLOP/s) or HBM (GB/s)
+};
+
+std::vector<Workload> workloads() {
+  const int64_t K4 = 4096, K8 = 8192;
+  return {
+      {"relu_f32_4096x4096", "imex_relu_f32", {K4 * K4},
+       {{Elem::F32, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}}, {K4 * K4}, false,
+       2.0 * K4 * K4 * 4, false},
+      {"silu_f32_512x640x20x15", "imex_silu_f32", {98304000},
+       {{Elem::F32, {98304000}, true, -8, 8}, {Elem::F32, {98304000}, false, 0, 0}}, {98304000}, false,
+       2.0 * 98304000 * 4, false},
+      {"softmax_f16_16384x1024", "imex_softmax_f16", {16384, 1024},
+       {{Elem::F16, {16384, 1024}, true, -4, 4}, {Elem::F16, {16384, 1024}, false, 0, 0}}, {16384, 1024}, false,
+       2.0 * 16384 * 1024 * 2, false},
+      {"rowsum_f32_8192x8192", "imex_rowsum_f32", {K8, K8},
+       {{Elem::F32, {K8, K8}, true, 0, 1}, {Elem::F32, {K8}, false, 0, 0}}, {K8, K8}, true,
+       K8 * K8 * 4.0 + K8 * 4.0, false},
+      {"transpose_bf16_8192x8192", "imex_transpose2d_b16", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, false,
+       2.0 * K8 * K8 * 2, false},
+      {"transpose_f32_4096x4096", "imex_transpose2d_b32", {K4, K4},
+       {{Elem::F32, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}}, {K4, K4}, false,
+       2.0 * K4 * K4 * 4, false},
+      {"gemm_f16_4096", "imex_gemm_f16_f16_f32", {K4, K4, K4},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, false, 2.0 * K4 * K4 * K4, true},
+      {"gemm_mlp_bf16_4096x11008x4096", "imex_gemm_bf16_bias_silu_bf16", {K4, 11008, K4},
+       {{Elem::BF16, {K4, K4}, true, -1.7f, 1.7f}, {Elem::BF16, {K4, 11008}, true, -0.035f, 0.035f},
+        {Elem::F32, {11008}, true, -0.17f, 0.17f}, {Elem::BF16, {K4, 11008}, false, 0, 0}},
+       {K4, 11008, K4}, false, 2.0 * K4 * 11008 * K4, true},
+  };
+}
+
+int64_t count(const Tensor &t) {
+  int64_t n = 1;
+  for (int64_t d : t.shape)
+    n *= d;
+  return n;
+}
+
+// Host fill through the runner utilities, on a rank-1 view of the buffer.
+void fillHost(void *host, const Tensor &t) {
+  struct Desc1D {
+    void *allocated, *aligned;
+    int64_t offset, size, stride;
+  } d = {host, host, 0, count(t), 1};
+  ImexUnrankedMemRef m = {1, &d};
+  switch (t.elem) {
+  case Elem::F32: _mlir_ciface_fillResource1DRandomF32(&m, t.lo, t.hi, false); break;
+  case Elem::F16: _mlir_ciface_fillResource1DRandomF16(&m, t.lo, t.hi, false); break;
+  case Elem::BF16: _mlir_ciface_fillResource1DRandomBF16(&m, t.lo, t.hi, false); break;
+  }
+}
+
+struct Options {
+  int runs = 100, warmups = 10, launchOnly = 0;
+  bool flush = false;
+};
+
+int runWorkload(const Workload &w, const Options &opt) {
+  void *stream = gpuCreateStream(nullptr, nullptr);
+  std::vector<void *> dev;
+  std::vector<std::vector<char>> host;
+  for (const Tensor &t : w.tensors) {
+    const size_t bytes = static_cast<size_t>(count(t)) * elemBytes(t.elem);
+    dev.push_back(gpuMemAlloc(stream, bytes, 64, /*isShared=*/0));
+    if (t.isInput) {
+      host.emplace_back(bytes);
+      fillHost(host.back().data(), t);
+      gpuMemCopy(stream, dev.back(), host.back().data(), bytes);
+    }
+  }
+
+  size_t grid[3], block[3], smem = 0;
+  if (imexHipKernelLaunchShape(w.kernel, w.dims.data(), static_cast<int>(w.dims.size()), grid, block, &smem) != 0) {
+    fprintf(stderr, "%s: no launch shape for %s\n", w.name, w.kernel);
+    return 1;
+  }
+  size_t blobSize = 0;
+  const void *blob = imexHipKernelModule(w.kernel, &blobSize);
+  void *module = gpuModuleLoad(stream, blob, blobSize);
+  void *kernel = gpuKernelGet(stream, module, w.kernel);
+
+  // ParamDesc list: pointers, then i64 scalars, then the optional f32 init; {NULL,0} ends it.
+  std::vector<int64_t> idx(w.indexArgs);
+  float init = 0.0f;
+  std::vector<ImexParamDesc> params;
+  for (void *&p : dev)
+    params.push_back({&p, sizeof(void *)});
+  for (int64_t &v : idx)
+    params.push_back({&v, sizeof(int64_t)});
+  if (w.hasInit)
+    params.push_back({&init, sizeof(float)});
+  params.push_back({nullptr, 0});
+  ImexEventDesc noDeps[1] = {{nullptr}};
+
+  if (opt.launchOnly > 0) {
+    for (int i = 0; i < opt.launchOnly; ++i)
+      gpuLaunchKernel(stream, kernel, grid[0], grid[1], grid[2], block[0], block[1], block[2], smem, params.data(),
+                      noDeps);
+    gpuWait(stream);
+    printf("%s: launched %s %d times, grid (%zu,%zu,%zu) block (%zu,%zu,%zu)\n", w.name, w.kernel, opt.launchOnly,
+           grid[0], grid[1], grid[2], block[0], block[1], block[2]);
+  } else {
+    std::vector<float> times(opt.runs);
+    imexHipProfileKernel(stream, kernel, grid[0], grid[1], grid[2], block[0], block[1], block[2], smem, params.data(),
+                         opt.warmups, opt.runs, opt.flush ? (size_t(512) << 20) : 0, 0, times.data());
+    float s[9];
+    imexHipComputeStats(times.data(), times.size(), s);
+    float total = 0.0f;
+    imexHipProfileKernel(stream, kernel, grid[0], grid[1], grid[2], block[0], block[1], block[2], smem, params.data(),
+                         opt.warmups, opt.runs, 0, 1, &total);
+    const double backToBackMs = total / opt.runs;
+    printf("%s: the kernel execution time is (ms, on HIP runtime):avg: %.4f, min: %.4f, max: %.4f, median: %4f, "
+           "std_deviation: %4f, variance: %4f, P95: %4f, P5: %4f, median_one_third_avg: %4f (over %d runs)\n",
+           w.name, s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], s[8], opt.runs);
+    const double rate = w.work / (backToBackMs * (w.mfma ? 1e9 : 1e6));
+    printf("%s: back-to-back %.4f ms/launch = %.1f %s (%.1f%% of the %s roofline)%s\n", w.name, backToBackMs, rate,
+           w.mfma ? "TFLOP/s" : "GB/s", 100.0 * rate / (w.mfma ? 2500.0 : 8000.0), w.mfma ? "2.5 PFLOP/s MFMA" : "8 TB/s HBM",
+           opt.flush ? " [per-launch times above measured after a cache flush]" : "");
+  }
+  fflush(stdout);
+
+  for (void *p : dev)
+    gpuMemFree(stream, p);
+  gpuStreamDestroy(stream);
+  return 0;
+}
+
+} // namespace
+
+int main(int argc, char **argv) {
+  Options opt;
+  std::vector<std::string> names;
+  const std::vector<Workload> all = workloads();
+  for (int i = 1; i < argc; ++i) {
+    const std::string a = argv[i];
+    if (a == "--list") {
+      for (const Workload &w : all)
+        printf("%s  (%s)\n", w.name, w.kernel);
+      return 0;
+    } else if (a == "-l") {
+      // backend selector of bench_imex; HIP is the only one here
+    } else if (a == "--flush") {
+      opt.flush = true;
+    } else if (a == "--runs" && i + 1 < argc) {
+      opt.runs = atoi(argv[++i]);
+    } else if (a == "--warmups" && i + 1 < argc) {
+      opt.warmups = atoi(argv[++i]);
+    } else if (a == "--launch-only" && i + 1 < argc) {
+      opt.launchOnly = atoi(argv[++i]);
+    } else if (a == "all") {
+      for (const Workload &w : all)
+        names.push_back(w.name);
+    } else {
+      names.push_back(a);
+    }
+  }
+  if (names.empty() || opt.runs < 1) {
+    fprintf(stderr, "usage: imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--launch-only N] <workload>|all ...\n"
+                    "       imex-hip-bench --list\n");
+    return 2;
+  }
+  printf("\n================ Imex Perf (HIP runtime) ================\n\n");
+  for (const std::string &n : names) {
+    const Workload *found = nullptr;
+    for (const Workload &w : all)
+      if (n == w.name)
+        found = &w;
+    if (!found) {
+      fprintf(stderr, "unknown workload %s (try --list)\n", n.c_str());
+      return 2;
+    }
+    if (int rc = runWorkload(*found, opt))
+      return rc;
+  }
+  return 0;
+}

@@ -15,8 +15,9 @@
 //    by blob address for the life of the process; kernels are cached per
 //    (module, name), so the load+get pair that precedes every launch costs two
 //    map lookups;
-//  * events returned by gpuLaunchKernel are owned by the stream and released
-//    when it is destroyed (the reference never frees them);
+//  * events returned by gpuLaunchKernel are stream positions, owned by the
+//    stream and released when it is destroyed (the reference never frees
+//    them); the HIP event behind one is recorded only when it is first used;
 //  * profiling uses hipEvent pairs on the launch stream.
 //
 //===----------------------------------------------------------------------===//
@@ -61,11 +62,27 @@ inline void checkHip(hipError_t res, const char *expr) {
 }
 #define CHECK_HIP(expr) checkHip((expr), #expr)
 
+struct GpuHipQueue;
+
+// What gpuLaunchKernel returns: a position in a stream (after the launch with
+// this sequence number).  No GPU-side marker is recorded at launch time -- a
+// completion signal per kernel costs ~15 us of dispatch bubble between
+// back-to-back launches, and host code that launches synchronously discards the
+// event anyway.  The HIP event is materialised on first use: recording it then
+// still places it after the launch it stands for (streams are in order), so a
+// dependency on it is satisfied no earlier than the reference semantics demand.
+struct LaunchEvent {
+  GpuHipQueue *queue;
+  uint64_t sequence;
+  hipEvent_t event; // null until someone waits on or times this position
+};
+
 struct GpuHipQueue {
   int device = 0;
   hipStream_t stream = nullptr;
   bool ownsStream = true;
-  std::vector<hipEvent_t> events; // handed out by gpuLaunchKernel
+  uint64_t launches = 0;
+  std::vector<LaunchEvent *> events; // handed out by gpuLaunchKernel / imexHipRecordTimestamp
   void *flushBuffer = nullptr;    // scratch for the profiler's cache flush
   size_t flushBytes = 0;
 
@@ -83,8 +100,11 @@ struct GpuHipQueue {
   ~GpuHipQueue() noexcept(false) {
     CHECK_HIP(hipSetDevice(device));
     CHECK_HIP(hipStreamSynchronize(stream));
-    for (hipEvent_t e : events)
-      CHECK_HIP(hipEventDestroy(e));
+    for (LaunchEvent *e : events) {
+      if (e->event)
+        CHECK_HIP(hipEventDestroy(e->event));
+      delete e;
+    }
     if (flushBuffer)
       CHECK_HIP(hipFree(flushBuffer));
     if (ownsStream)
@@ -361,17 +381,32 @@ long envLong(const char *name, long fallback) {
   return fallback;
 }
 
-hipEvent_t launchKernel(GpuHipQueue *queue, void *kernel, size_t gx, size_t gy, size_t gz, size_t bx,
-                        size_t by, size_t bz, size_t sharedMemBytes, ImexParamDesc *params,
-                        ImexEventDesc *depEvents) {
+hipEvent_t materialise(LaunchEvent *le) {
+  if (!le->event) {
+    CHECK_HIP(hipSetDevice(le->queue->device));
+    CHECK_HIP(hipEventCreate(&le->event));
+    CHECK_HIP(hipEventRecord(le->event, le->queue->stream));
+  }
+  return le->event;
+}
+
+LaunchEvent *launchKernel(GpuHipQueue *queue, void *kernel, size_t gx, size_t gy, size_t gz, size_t bx,
+                          size_t by, size_t bz, size_t sharedMemBytes, ImexParamDesc *params,
+                          ImexEventDesc *depEvents) {
   if (!queue)
     throw std::runtime_error("gpuLaunchKernel: null stream");
   LaunchArgs la = makeLaunch(kernel, gx, gy, gz, bx, by, bz, sharedMemBytes, params);
-  CHECK_HIP(hipSetDevice(queue->device));
 
   size_t depCount = countUntil(depEvents, [](const ImexEventDesc &e) { return e.event == nullptr; });
-  for (size_t i = 0; i < depCount; ++i)
-    CHECK_HIP(hipStreamWaitEvent(queue->stream, static_cast<hipEvent_t>(depEvents[i].event), 0));
+  for (size_t i = 0; i < depCount; ++i) {
+    LaunchEvent *dep = static_cast<LaunchEvent *>(depEvents[i].event);
+    if (dep->queue == queue)
+      continue; // same in-order stream: already ordered
+    hipEvent_t ev = materialise(dep);
+    CHECK_HIP(hipSetDevice(queue->device));
+    CHECK_HIP(hipStreamWaitEvent(queue->stream, ev, 0));
+  }
+  CHECK_HIP(hipSetDevice(queue->device));
 
   if (getenv("IMEX_ENABLE_PROFILING")) {
     // Defaults of LevelZeroRuntimeWrappers.cpp:521-523; a positive
@@ -396,9 +431,7 @@ hipEvent_t launchKernel(GpuHipQueue *queue, void *kernel, size_t gx, size_t gy, 
   }
 
   enqueue(queue, la);
-  hipEvent_t done;
-  CHECK_HIP(hipEventCreate(&done));
-  CHECK_HIP(hipEventRecord(done, queue->stream));
+  LaunchEvent *done = new LaunchEvent{queue, ++queue->launches, nullptr};
   queue->events.push_back(done);
   return done;
 }
@@ -565,13 +598,27 @@ extern "C" int imexHipProfileKernel(void *queue, void *kernel, size_t gridX, siz
   });
 }
 
+extern "C" void *imexHipRecordTimestamp(void *queue) {
+  return catchAll([&]() -> void * {
+    if (!queue)
+      throw std::runtime_error("imexHipRecordTimestamp: null stream");
+    GpuHipQueue *q = asQueue(queue);
+    LaunchEvent *le = new LaunchEvent{q, q->launches, nullptr};
+    q->events.push_back(le);
+    materialise(le);
+    return le;
+  });
+}
+
 extern "C" float imexHipEventElapsedMs(void *startEvent, void *stopEvent) {
   return catchAll([&]() {
     if (!startEvent || !stopEvent)
       throw std::runtime_error("imexHipEventElapsedMs: null event");
+    hipEvent_t a = materialise(static_cast<LaunchEvent *>(startEvent));
+    hipEvent_t b = materialise(static_cast<LaunchEvent *>(stopEvent));
     float ms = 0.0f;
-    CHECK_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stopEvent)));
-    CHECK_HIP(hipEventElapsedTime(&ms, static_cast<hipEvent_t>(startEvent), static_cast<hipEvent_t>(stopEvent)));
+    CHECK_HIP(hipEventSynchronize(b));
+    CHECK_HIP(hipEventElapsedTime(&ms, a, b));
     return ms;
   });
 }

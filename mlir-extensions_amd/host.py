@@ -67,6 +67,7 @@ _RUNTIME_SYMBOLS = {
     "mgpuModuleUnload": (None, [C.c_void_p]),
     "imexHipProfileKernel": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_size_t] * 7 +
                              [C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_int, C.POINTER(C.c_float)]),
+    "imexHipRecordTimestamp": (C.c_void_p, [C.c_void_p]),
     "imexHipEventElapsedMs": (C.c_float, [C.c_void_p, C.c_void_p]),
     "imexHipComputeStats": (None, [C.POINTER(C.c_float), C.c_size_t, C.POINTER(C.c_float)]),
     "imexHipDeviceInfo": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_size_t),
@@ -240,6 +241,24 @@ class Stream:
         del keep
         return ev
 
+    def prepare(self, name, dims, args):
+        """Resolve the kernel, its launch shape and its ParamDesc list once and
+        return a zero-argument callable that performs just the gpuLaunchKernel
+        call (what JIT'd host code does inside a loop)."""
+        grid, block, smem = launch_shape(name, dims)
+        if 0 in grid:
+            return lambda: None
+        fn = self.kernel(name)
+        descs, keep = _pack_params(args)
+        params = C.cast(descs, C.c_void_p)
+        launch, handle = self.rt.gpuLaunchKernel, self.handle
+        gx, gy, gz = grid
+        bx, by, bz = block
+
+        def run(_keep=(descs, keep)):
+            return launch(handle, fn, gx, gy, gz, bx, by, bz, smem, params, None)
+        return run
+
     def profile(self, name, dims, args, warmups=5, rounds=20, flush_bytes=0, mode=0):
         """Per-launch times in ms (mode 0) or [total ms] over `rounds` back-to-back launches (mode 1)."""
         grid, block, smem = launch_shape(name, dims)
@@ -254,6 +273,9 @@ class Stream:
 
     def wait(self):
         self.rt.gpuWait(self.handle)
+
+    def timestamp(self):
+        return self.rt.imexHipRecordTimestamp(self.handle)
 
     def elapsed_ms(self, start_event, stop_event):
         return self.rt.imexHipEventElapsedMs(start_event, stop_event)

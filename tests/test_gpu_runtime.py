@@ -88,7 +88,10 @@ def test_event_dependencies_across_streams(host, orc):
         s2.wait()
         got = s2.from_device(d_out, (n,), np.float32)
         assert np.array_equal(got, orc.relu_f32(orc.silu_f32(x)))
-        assert s1.elapsed_ms(ev, ev) == 0.0
+        t0 = s1.timestamp()
+        s1.launch("imex_silu_f32", [n], [d_in, d_mid, n])
+        t1 = s1.timestamp()
+        assert 0.0 < s1.elapsed_ms(t0, t1) < 100.0
         for p in (d_in, d_mid, d_out):
             s1.free(p)
 
