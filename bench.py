@@ -194,8 +194,8 @@ def measure_secondary(stream, w, rounds):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--only", type=str, default=None, help="comma-separated workload names")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline legs")
     args = ap.parse_args()
@@ -231,6 +231,23 @@ def main():
     stream.free(d_probe)
     log("gpuMemCopy host->device: %.1f GB/s" % h2d_gbs)
 
+    # The secondary workloads run first: the device then enters the headline loop
+    # from a loaded state.  Coming from idle, the first ~100 GEMM launches run
+    # ~10% slower while the power controller settles, which a short timed region
+    # would mostly measure.
+    per = []
+    secondary = sorted(workloads[1:], key=lambda w: w.bound == "mfma")  # the other GEMM goes last
+    for w in secondary:
+        hot_ms, cold_ms = measure_secondary(stream, w, rounds=50)
+        rf = roofline(w, hot_ms)
+        entry_ = {"name": w.name, "workload": w.describe, "kernel": w.kernel, "dtype": w.dtype,
+                  "ms_per_launch": round(hot_ms, 5), "ms_per_launch_cache_flushed": round(cold_ms, 5),
+                  "roofline": rf, "roofline_cache_flushed": roofline(w, cold_ms)}
+        log("%s: %.4f ms (%.1f %s, %.1f%% of peak); cache-flushed %.4f ms (%.1f%%)" % (
+            w.name, hot_ms, rf["achieved"], rf["unit"], 100 * rf["frac"], cold_ms,
+            100 * entry_["roofline_cache_flushed"]["frac"]))
+        per.append(entry_)
+
     head = workloads[0]
     K, W = args.steps, args.warmup
     step = stream.prepare(head.kernel, head.dims, head.args)
@@ -259,8 +276,9 @@ def main():
                    "launch": "grid (256,1,1) x block (512,1,1)", "device": info["name"],
                    "cus": info["cus"], "clock_mhz": info["clock_khz"] / 1e3,
                    "gpuMemCopy_h2d_GBps": round(h2d_gbs, 1)},
-        "roofline": dict(roofline(head, kernel_ms), event_ms_per_step=round(event_ms, 5),
-                         kernel_ms=round(kernel_ms, 5)),
+        # `achieved` prices the launch at its HIP-event duration over the timed region
+        "roofline": dict(roofline(head, event_ms), event_ms_per_step=round(event_ms, 5),
+                         back_to_back_ms=round(kernel_ms, 5)),
     }
 
     if not args.no_cpu and head.cpu:
@@ -270,22 +288,12 @@ def main():
                                   "sample": sample, "host_cores": os.cpu_count()}
         log("cpu baseline %s: %.4f GFLOP/s (%.1f s)" % (head.name, v * 1e3, time.time() - t))
 
-    per = []
-    for w in workloads[1:]:
-        hot_ms, cold_ms = measure_secondary(stream, w, rounds=50)
-        rf = roofline(w, hot_ms)
-        entry_ = {"name": w.name, "workload": w.describe, "kernel": w.kernel, "dtype": w.dtype,
-                  "ms_per_launch": round(hot_ms, 5), "ms_per_launch_cache_flushed": round(cold_ms, 5),
-                  "roofline": rf, "roofline_cache_flushed": roofline(w, cold_ms)}
-        log("%s: %.4f ms (%.1f %s, %.1f%% of peak); cache-flushed %.4f ms (%.1f%%)" % (
-            w.name, hot_ms, rf["achieved"], rf["unit"], 100 * rf["frac"], cold_ms,
-            100 * entry_["roofline_cache_flushed"]["frac"]))
+    for w, entry_ in zip(secondary, per):
         if not args.no_cpu and w.cpu:
             t = time.time()
             v, sample = w.cpu()
             entry_["cpu_baseline"] = {"value": round(v, 6), "unit": w.unit, "cores": 1, "kind": "port", "sample": sample}
             log("cpu baseline %s: %.4f %s (%.1f s)" % (w.name, v, w.unit, time.time() - t))
-        per.append(entry_)
     result["per_config"] = per
 
     for w in workloads:
