@@ -244,6 +244,10 @@ void oracle_silu_f32(const float *x, float *y, size_t n) {
 
 float oracle_expf_cr(float x) { return (float)exp((double)x); }
 
+void oracle_expf_n(const float *in, float *out, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = expf(in[i]);
+}
+
 /* ======================================================================== */
 /* Softmax                                                                    */
 /* ======================================================================== */

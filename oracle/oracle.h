@@ -15,7 +15,7 @@
  * Pinning status (what independent evidence each function is tested against):
  *   relu, softmax, row-sum, transpose, gemm (f32 / f16 / bf16 inputs), bias add,
  *   half->float, bfloat->float, allclose, stats   : reference golden vectors
- *       and closed forms (tests/golden, tests/test_oracle_*.py);
+ *       and closed forms (tests/golden, tests/test_oracle.py);
  *   stats (reference median formula)              : also the reference's own
  *       ExecutionEngineUtils.cpp compiled into oracle/_ref;
  *   float->half / float->bfloat rounding          : exhaustive comparison with
@@ -63,6 +63,7 @@ void oracle_relu_olt_f32(const float *x, float *y, size_t n);          /* test/P
 void oracle_silu_f32(const float *x, float *y, size_t n);              /* benchmarks/silu/silu_gpu.mlir.in:8-18 */
 float oracle_silu_scalar_f32(float x);
 float oracle_expf_cr(float x);                                          /* correctly rounded exp via f64 */
+void oracle_expf_n(const float *in, float *out, size_t n);              /* the host libm expf the oracle's silu/softmax call */
 
 /* ---- softmax --------------------------------------------------------------- */
 void oracle_softmax_f32(const float *x, float *y, int64_t rows, int64_t cols);        /* benchmarks/softmax/softmax_gpu.mlir.in:4-44 */
