@@ -13,10 +13,12 @@
 // runtime):avg: ..." line per workload, the line bench_imex greps into
 // report.txt (bench_imex.in:87-91).
 //
-//   imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--launch-only N] <workload>...
+//   imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--launch-only N] <workload>...
 //   imex-hip-bench --list
 //
 //   -l             accepted for bench_imex compatibility (the HIP runtime is the only backend here)
+//   --zeros        all-zero inputs instead of random ones: MFMA power, and with it the clock the
+//                  part sustains, depends on operand values; this shows the kernel at full clock
 //   --launch-only  skip the timing loop and just launch the kernel N times (for
 //                  rocprofv3 counter runs, which time and count every dispatch themselves)
 //
@@ -109,7 +111,7 @@ void fillHost(void *host, const Tensor &t) {
 
 struct Options {
   int runs = 100, warmups = 10, launchOnly = 0;
-  bool flush = false;
+  bool flush = false, zeros = false;
 };
 
 int runWorkload(const Workload &w, const Options &opt) {
@@ -121,7 +123,8 @@ int runWorkload(const Workload &w, const Options &opt) {
     dev.push_back(gpuMemAlloc(stream, bytes, 64, /*isShared=*/0));
     if (t.isInput) {
       host.emplace_back(bytes);
-      fillHost(host.back().data(), t);
+      if (!opt.zeros)
+        fillHost(host.back().data(), t);
       gpuMemCopy(stream, dev.back(), host.back().data(), bytes);
     }
   }
@@ -172,7 +175,7 @@ int runWorkload(const Workload &w, const Options &opt) {
     const double rate = w.work / (backToBackMs * (w.mfma ? 1e9 : 1e6));
     printf("%s: back-to-back %.4f ms/launch = %.1f %s (%.1f%% of the %s roofline)%s\n", w.name, backToBackMs, rate,
            w.mfma ? "TFLOP/s" : "GB/s", 100.0 * rate / (w.mfma ? 2500.0 : 8000.0), w.mfma ? "2.5 PFLOP/s MFMA" : "8 TB/s HBM",
-           opt.flush ? " [per-launch times above measured after a cache flush]" : "");
+           opt.flush ? " [per-launch times above measured after a cache flush]" : (opt.zeros ? " [all-zero inputs]" : ""));
   }
   fflush(stdout);
 
@@ -198,6 +201,8 @@ int main(int argc, char **argv) {
       // backend selector of bench_imex; HIP is the only one here
     } else if (a == "--flush") {
       opt.flush = true;
+    } else if (a == "--zeros") {
+      opt.zeros = true;
     } else if (a == "--runs" && i + 1 < argc) {
       opt.runs = atoi(argv[++i]);
     } else if (a == "--warmups" && i + 1 < argc) {
@@ -212,7 +217,7 @@ int main(int argc, char **argv) {
     }
   }
   if (names.empty() || opt.runs < 1) {
-    fprintf(stderr, "usage: imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--launch-only N] <workload>|all ...\n"
+    fprintf(stderr, "usage: imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--launch-only N] <workload>|all ...\n"
                     "       imex-hip-bench --list\n");
     return 2;
   }

@@ -10,26 +10,29 @@
 //   benchmarks/silu/silu_gpu.mlir.in:3-19 for the activation fused below.
 //
 // Blocking on MI355X:
-//   workgroup tile 256 x 256, K-step 64, 512 threads = 8 wavefronts in a 2 x 4
-//   grid (two per SIMD), each owning 128 x 64 = 4 x 2 MFMA 32x32x16 tiles;
-//   A and B tiles go from global memory STRAIGHT into LDS (buffer_load ... lds,
-//   16 bytes per lane, no register staging), double-buffered: the copies for
-//   step k+1 are issued at the top of step k and awaited just before the
-//   step's single barrier;
-//   the LDS images are swizzled -- A [256 rows][64 k] by 16-byte group, B
-//   [64 k][256 n] by 32-byte pair -- and because a direct copy fixes each lane's
+//   workgroup tile 256 x 256, 512 threads = 8 wavefronts in a 2 x 4 grid (two per
+//   SIMD), each owning 128 x 64 = 4 x 2 MFMA 32x32x16 tiles (128 accumulator
+//   registers);
+//   K advances 32 at a time through a ring of four 32 KiB LDS stages: A and B
+//   tiles go from global memory STRAIGHT into LDS (buffer_load ... lds, 16 bytes
+//   per lane, no register staging) three steps ahead of the step that multiplies
+//   them; a step waits (vmcnt) only for the oldest tile in flight, then meets the
+//   other wavefronts at the step's single barrier;
+//   the LDS images are swizzled -- A [256 rows][32 k] by 16-byte group, B
+//   [32 k][256 n] by 32-byte pair -- and because a direct copy fixes each lane's
 //   LDS position, the swizzle is applied to the lane's GLOBAL address instead;
 //   A fragments are 128-bit LDS reads; B is row-major [K,N] while the MFMA wants
 //   eight consecutive k per lane, so B fragments use the LDS transpose read
-//   (ds_read_b64_tr_b16) -- no permutes, no transposed writes; neither side has
-//   LDS bank conflicts (SQ_LDS_BANK_CONFLICT = 0);
-//   fragments are double-buffered in registers: the LDS reads of slice s+1 run
-//   under the MFMAs of slice s (sched_group_barrier pins the interleaving);
+//   (ds_read_b64_tr_b16) -- no permutes, no transposed copy of B anywhere;
+//   fragments are double-buffered in registers: the LDS reads of slice s+1 are
+//   placed by hand between the MFMAs of slice s (sched_barrier fences keep the
+//   order), and the barrier sits between a step's two slices so that eight
+//   MFMAs are always queued behind it;
 //   workgroup ids are remapped so that the 32 workgroups resident on one XCD
 //   (ids congruent mod 8) cover a compact 4 x 8 block of tiles and share A and
-//   B panels in that XCD's L2 (L2 hit rate 78%, fabric fetch 1.5x the minimum).
+//   B panels in that XCD's L2.
 //
-// Shapes that are not multiples of the tile (M%256, N%256, K%64) take the
+// Shapes that are not multiples of the tile (M%256, N%256, K%32) take the
 // one-thread-per-output path of the same kernels, which adds in ascending k
 // like the reference's CPU loop (lib/ExecutionEngine/ImexRunnerUtils.cpp:308-317).
 //
@@ -43,23 +46,22 @@ using namespace imexhip;
 
 namespace {
 
-// Wavefront grid inside the 256 x 256 workgroup tile: 2 x 4 (eight wavefronts,
-// two per SIMD, each 128 x 64) or 2 x 2 (four wavefronts, each 128 x 128).
-#ifndef IMEX_GEMM_WAVES_N
-#define IMEX_GEMM_WAVES_N 4
-#endif
-constexpr int kWavesM = 2, kWavesN = IMEX_GEMM_WAVES_N;
-constexpr int kThreads = 64 * kWavesM * kWavesN;
-constexpr int BM = 256, BN = 256, BK = 64;
+// Wavefront grid inside the 256 x 256 workgroup tile: 2 x 4, each wavefront 128 x 64.
+constexpr int kWavesM = 2, kWavesN = 4;
+constexpr int kWaves = kWavesM * kWavesN;
+constexpr int kThreads = 64 * kWaves;
+constexpr int BM = 256, BN = 256;
+constexpr int RK = 32;                              // K per step (one ring stage)
 constexpr int WM = BM / kWavesM, WN = BN / kWavesN; // wavefront tile
 constexpr int TI = WM / 32, TJ = WN / 32;           // MFMA 32x32 tiles per wavefront
-constexpr int kWaves = kWavesM * kWavesN;
-constexpr int kADma = BM * BK * 2 / 1024 / kWaves;  // 1 KiB global->LDS copies per wavefront and K-step (A)
-constexpr int kBDma = BK * BN * 2 / 1024 / kWaves;  // ... (B)
-constexpr int kABytes = BM * BK * 2;                // A image: [256 rows][64 k], 16-byte groups swizzled
-constexpr int kBBytes = BK * BN * 2;                // B image: [64 k][256 n], 32-byte pairs swizzled
-constexpr int kStageBytes = kABytes + kBBytes;     // 64 KiB; two stages = 128 KiB of the 160 KiB LDS
-constexpr int kGroupM = 4;                         // tile rows per L2-sharing group
+constexpr int kStages = 4;                          // LDS ring: 4 x 32 KiB of the 160 KiB
+constexpr int kRA = BM * RK * 2;                    // A image [256 rows][32 k], 16-byte groups swizzled
+constexpr int kRB = RK * BN * 2;                    // B image [32 k][256 n], 32-byte pairs swizzled
+constexpr int kRStage = kRA + kRB;
+constexpr int kRADma = kRA / 1024 / kWaves;         // 1 KiB global->LDS copies per wavefront and step (A)
+constexpr int kRBDma = kRB / 1024 / kWaves;         // ... (B)
+constexpr int kDist = kStages - 1;                  // tiles in flight ahead of the one being multiplied
+constexpr int kGroupM = 4;                          // tile rows per L2-sharing group
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -67,9 +69,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) i16x4 LdsI16x4; // operand type of the LDS transpose read
 typedef __attribute__((address_space(3))) char LdsChar;
-
-struct Stage0 { static constexpr int value = 0; };
-struct Stage1 { static constexpr int value = 1; };
 
 struct F16 {
   using Frag = f16x8;
@@ -86,29 +85,8 @@ struct BF16 {
   static __device__ __forceinline__ float widen(uint16_t h) { return bf16_bits_to_float(h); }
 };
 
-// Byte offset of 16-byte group `chunk` (0..7) of row `row` in a [rows][64]
-// 16-bit LDS image.  The xor spreads both "same chunk, consecutive rows"
-// (fragment reads) and "same chunk, rows 8 apart" (transposed B writes) over
-// all banks.
-__device__ __forceinline__ int lds_off(int row, int chunk) {
-  return row * (BK * 2) + (((chunk ^ row ^ (row >> 3)) & 7) << 4);
-}
-
-// Instruction-class masks of __builtin_amdgcn_sched_group_barrier.
-#define IMEX_SG(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-#define IMEX_MFMA 0x008
-#define IMEX_VALU 0x002
-#define IMEX_VMEM_RD 0x020
-#define IMEX_DS_RD 0x100
-#define IMEX_DS_WR 0x200
-#define IMEX_REP4(x) x x x x
-#if IMEX_GEMM_WAVES_N == 2
-// per slice: 16 MFMAs and 12 LDS reads (4 b128 for A, 8 transpose reads for B)
-#define IMEX_SCHED_SLICE() IMEX_REP4(IMEX_SG(IMEX_MFMA, 1); IMEX_SG(IMEX_DS_RD, 1); IMEX_SG(IMEX_MFMA, 1); IMEX_SG(IMEX_DS_RD, 1); IMEX_SG(IMEX_MFMA, 1); IMEX_SG(IMEX_DS_RD, 1); IMEX_SG(IMEX_MFMA, 1);)
-#else
-// per slice: 8 MFMAs and 8 LDS reads (4 b128 for A, 4 transpose reads for B)
-#define IMEX_SCHED_SLICE() IMEX_REP4(IMEX_SG(IMEX_MFMA, 1); IMEX_SG(IMEX_DS_RD, 1); IMEX_SG(IMEX_MFMA, 1); IMEX_SG(IMEX_DS_RD, 1);)
-#endif
+// Keeps the compiler's scheduler from moving anything across this point.
+#define IMEX_FENCE() __builtin_amdgcn_sched_barrier(0)
 
 // ---- epilogues ------------------------------------------------------------------
 struct StoreF32 {       // C = acc
@@ -150,16 +128,18 @@ struct StoreF16 {       // C(f16) = acc   (WG/gemm_4kx4kx4k_f16_f16_f16.mlir)
 template <typename T, typename Epi>
 __device__ __forceinline__ void gemm_scalar(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
                                             Epi epi) {
-  const int64_t idx = int64_t(blockIdx.x) * kThreads + threadIdx.x;
-  if (idx >= M * N)
-    return;
-  const int64_t m = idx / N, n = idx % N;
-  float acc = 0.0f;
-  for (int64_t k = 0; k < K; ++k) {
-    const float p = T::widen(A[m * K + k]) * T::widen(B[k * N + n]);
-    acc = acc + p; // rounded multiply, rounded add (file is built with contraction off)
+  // grid-stride, so that any launch shape covers every output
+  const int64_t block = int64_t(blockIdx.y) * gridDim.x + blockIdx.x;
+  const int64_t stride = int64_t(gridDim.x) * gridDim.y * kThreads;
+  for (int64_t idx = block * kThreads + threadIdx.x; idx < M * N; idx += stride) {
+    const int64_t m = idx / N, n = idx % N;
+    float acc = 0.0f;
+    for (int64_t k = 0; k < K; ++k) {
+      const float p = T::widen(A[m * K + k]) * T::widen(B[k * N + n]);
+      acc = acc + p; // rounded multiply, rounded add (file is built with contraction off)
+    }
+    epi(m, n, N, acc);
   }
-  epi(m, n, N, acc);
 }
 
 // ---- tiled MFMA path ----------------------------------------------------------------
@@ -170,21 +150,29 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, in
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, range, 0x00020000);
 }
 
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+
 template <typename T, typename Epi>
 __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                            int64_t M, int64_t N, int64_t K, Epi epi, char *lds) {
+  static_assert(TI == 4 && TJ == 2 && kWaves == 8, "written for 8 wavefronts of 4 x 2 MFMA tiles");
   LdsChar *lds_base = (LdsChar *)lds;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave / kWavesN, wn = wave % kWavesN;
 
-  // -- workgroup id -> tile, XCD-aware ------------------------------------------------
   const int tilesM = int(M / BM), tilesN = int(N / BN);
   const int tiles = tilesM * tilesN;
   int pid = blockIdx.y * gridDim.x + blockIdx.x;
+  if (pid >= tiles)
+    return; // a launch with more workgroups than tiles: the surplus has nothing to do
   if (tiles % 8 == 0)
-    pid = (pid % 8) * (tiles / 8) + pid / 8; // ids congruent mod 8 share an XCD
+    pid = (pid % 8) * (tiles / 8) + pid / 8;
   const int group = kGroupM * tilesN;
   const int firstM = (pid / group) * kGroupM;
   const int groupRows = min(tilesM - firstM, kGroupM);
@@ -192,67 +180,51 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
   const int tileN = (pid % group) / groupRows;
   const int64_t m0 = int64_t(tileM) * BM, n0 = int64_t(tileN) * BN;
 
-  // -- global -> LDS, directly (no register staging) ------------------------------------
-  // buffer_load_dwordx4 ... lds: each wavefront-level instruction moves 64 x 16 B
-  // from global memory into 1 KiB of contiguous LDS (lane l lands at base + 16 l;
-  // the LDS base is wave-uniform, in M0).  The LDS images are swizzled, so the
-  // swizzle is applied on the GLOBAL side: a lane fetches the piece that belongs
-  // at its fixed LDS position.
-  //   A image [256 rows][64 k]: one instruction = 8 rows; 16-byte group c of row r
-  //     lives at group c ^ ((r ^ r>>3) & 7).
-  //   B image [64 k][256 n] (row-major, 512 B rows): one instruction = 2 k rows; the
-  //     32-byte pair p of row r lives at pair p ^ g(r), g(r) = (r & 3) | ((r>>3 & 1) << 2),
-  //     which spreads the rows a transpose read touches over all LDS banks.
+  // global -> LDS copies.  A image: 64-byte rows, 16-byte group c of row r stored at
+  // group c ^ ((r >> 2) & 3); one copy = 16 rows.  B image: 512-byte rows, 32-byte pair p
+  // of row r at pair p ^ g(r); one copy = 2 rows.
   const int waveU = __builtin_amdgcn_readfirstlane(wave);
   const __amdgpu_buffer_rsrc_t aRsrc = make_rsrc(A + m0 * K, int64_t(BM) * K * 2);
   const __amdgpu_buffer_rsrc_t bRsrc = make_rsrc(B + n0, (K * N - n0) * 2);
-  int aVoff[kADma], bVoff[kBDma];
+  int aVoff[kRADma], bVoff[kRBDma];
 #pragma unroll
-  for (int q = 0; q < kADma; ++q) {
-    const int row = wave * (BM / kWaves) + q * 8 + (lane >> 3);
-    const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
+  for (int q = 0; q < kRADma; ++q) {
+    const int row = wave * (BM / kWaves) + q * 16 + (lane >> 2);
+    const int chunk = (lane & 3) ^ ((row >> 2) & 3);
     aVoff[q] = int((int64_t(row) * K + chunk * 8) * 2);
   }
 #pragma unroll
-  for (int q = 0; q < kBDma; ++q) {
-    const int row = wave * (BK / kWaves) + q * 2 + (lane >> 5);
+  for (int q = 0; q < kRBDma; ++q) {
+    const int row = wave * (RK / kWaves) + q * 2 + (lane >> 5);
     const int g = (row & 3) | (((row >> 3) & 1) << 2);
     const int chunk = (((((lane & 31) >> 1) ^ g)) << 1) | (lane & 1);
     bVoff[q] = int((int64_t(row) * N + chunk * 8) * 2);
   }
-  const int bStep = int(BK * N * 2); // bytes of B per K-step
-  auto dma_tile = [&](int kt, int stage) {
-    LdsChar *aDst = reinterpret_cast<LdsChar *>(lds_base) + stage * kStageBytes + waveU * (BM / kWaves) * 128;
-    LdsChar *bDst = reinterpret_cast<LdsChar *>(lds_base) + stage * kStageBytes + kABytes + waveU * (BK / kWaves) * 512;
+  const int bStep = int(RK * N * 2);
+  auto dma_tile = [&](int kt, int stageOff) { // stageOff = byte offset of the stage, wave-uniform
+    LdsChar *aDst = lds_base + stageOff + waveU * (BM / kWaves) * (RK * 2);
+    LdsChar *bDst = lds_base + stageOff + kRA + waveU * (RK / kWaves) * 512;
 #pragma unroll
-    for (int q = 0; q < kADma; ++q)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(aRsrc, aDst + q * 1024, 16, aVoff[q], kt * (BK * 2), 0, 0);
+    for (int q = 0; q < kRADma; ++q)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(aRsrc, aDst + q * 1024, 16, aVoff[q], kt * (RK * 2), 0, 0);
 #pragma unroll
-    for (int q = 0; q < kBDma; ++q)
+    for (int q = 0; q < kRBDma; ++q)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(bRsrc, bDst + q * 1024, 16, bVoff[q], kt * bStep, 0, 0);
   };
 
-  // -- LDS -> MFMA fragments ---------------------------------------------------------------
-  // A: ds_read_b128 of row w*WM + i*32 + (lane&31), 16-byte group ks*2 + (lane>>5).  The
-  // swizzled position is ((ks*2 ^ (i&1)*4) ^ z) with z per lane, so four per-lane
-  // bases (c = 0,2,4,6) serve every (i, ks); the rest is an immediate.
   const int fragRow = lane & 31, fragHalf = lane >> 5;
-  int aRd[4];
+  int aRd[2];
 #pragma unroll
-  for (int c = 0; c < 4; ++c)
-    aRd[c] = lds_off(wm * WM + fragRow, 2 * c + fragHalf);
-  // B: LDS transpose read (ds_read_b64_tr_b16).  Within each group of 16 lanes,
-  // lane t supplies the address of 4 consecutive n at k row t/4 and receives 4
-  // consecutive k of column n = t.  Lanes 0-31 cover k 0-7 of the slice, lanes
-  // 32-63 k 8-15; two reads (k +0..3, +4..7) make one 8-wide MFMA operand.
+  for (int ks = 0; ks < 2; ++ks)
+    aRd[ks] = (wm * WM + fragRow) * (RK * 2) + ((((ks * 2 + fragHalf) ^ (fragRow >> 2)) & 3) << 4);
   int bRd[TJ];
   {
     const int t = lane & 15, nblock = (lane >> 4) & 1, khalf = lane >> 5;
-    const int g = (t >> 2) | (khalf << 2);                 // g(row) for row = ks*16 + khalf*8 + h*4 + t/4
-    const int pair0 = (wn * WN) / 16 + nblock;             // 32-byte pair holding this lane's n, tile j = 0
+    const int g = (t >> 2) | (khalf << 2);
+    const int pair0 = (wn * WN) / 16 + nblock;
 #pragma unroll
     for (int j = 0; j < TJ; ++j)
-      bRd[j] = kABytes + (khalf * 8 + (t >> 2)) * 512 + (((pair0 + 2 * j) ^ g) * 32) + (t & 3) * 8;
+      bRd[j] = kRA + (khalf * 8 + (t >> 2)) * 512 + (((pair0 + 2 * j) ^ g) * 32) + (t & 3) * 8;
   }
 
   f32x16 acc[TI][TJ];
@@ -265,69 +237,63 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
         acc[i][j][r] = 0.0f;
 
   typename T::Frag af[2][TI], bf[2][TJ];
-  auto read_frags = [&](int stage, int ks, int buf) {
-    const char *base = lds + stage * kStageBytes;
-#pragma unroll
-    for (int i = 0; i < TI; ++i) {
-      const int c = (ks ^ ((i & 1) << 1)) & 3; // which per-lane base: (ks*2 ^ (i&1)*4) / 2
-      af[buf][i] = *reinterpret_cast<const typename T::Frag *>(base + aRd[c] + i * 32 * 128);
-    }
-#pragma unroll
-    for (int j = 0; j < TJ; ++j) {
-      const char *p = base + bRd[j] + ks * 16 * 512;
-      const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p));
-      const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p + 4 * 512));
-      bf[buf][j] = __builtin_bit_cast(typename T::Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-    }
+  auto read_a = [&](int stageOff, int ks, int buf, int i) {
+    af[buf][i] = *reinterpret_cast<const typename T::Frag *>(lds + stageOff + aRd[ks] + i * 32 * (RK * 2));
   };
-  auto mfma_slice = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < TI; ++i)
-#pragma unroll
-      for (int j = 0; j < TJ; ++j)
-        acc[i][j] = T::mfma(af[buf][i], bf[buf][j], acc[i][j]);
+  auto read_b = [&](int stageOff, int ks, int buf, int j) {
+    const char *p = lds + stageOff + bRd[j] + ks * 16 * 512;
+    const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p));
+    const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p + 4 * 512));
+    bf[buf][j] = __builtin_bit_cast(typename T::Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+  auto mm = [&](int buf, int i, int j) { acc[i][j] = T::mfma(af[buf][i], bf[buf][j], acc[i][j]); };
+  // 8 MFMAs from register buffer `buf`, interleaved with the 8 LDS reads that fill buf^1
+  auto slice = [&](int buf, int rOff, int rks) {
+    mm(buf, 0, 0); read_a(rOff, rks, buf ^ 1, 0); IMEX_FENCE();
+    mm(buf, 0, 1); read_a(rOff, rks, buf ^ 1, 1); IMEX_FENCE();
+    mm(buf, 1, 0); read_b(rOff, rks, buf ^ 1, 0); IMEX_FENCE();
+    mm(buf, 1, 1); read_a(rOff, rks, buf ^ 1, 2); IMEX_FENCE();
+    mm(buf, 2, 0); read_a(rOff, rks, buf ^ 1, 3); IMEX_FENCE();
+    mm(buf, 2, 1); read_b(rOff, rks, buf ^ 1, 1); IMEX_FENCE();
+    mm(buf, 3, 0); IMEX_FENCE();
+    mm(buf, 3, 1); IMEX_FENCE();
   };
 
-  // One K-step = four 16-wide slices; fragments are double-buffered in
-  // registers (the reads of slice s+1 run under the MFMAs of slice s).  The
-  // asynchronous copies of tile kt+1 into the other LDS stage are issued at the
-  // top of step kt and awaited (vmcnt) just before the step's closing barrier.
-  // Past the end of K they re-fetch the last tile into the stage nobody reads, so
-  // every step is the same branch-free code.
-  const int kTiles = int(K / BK);
+  const int kTiles = int(K / RK);
   const int lastTile = kTiles - 1;
-  auto k_step = [&](int kt, auto stageTag) {
-    constexpr int cur = decltype(stageTag)::value;
-    dma_tile(min(kt + 1, lastTile), cur ^ 1);
-    read_frags(cur, 1, 1);
-    mfma_slice(0);
-    IMEX_SCHED_SLICE();
-    read_frags(cur, 2, 0);
-    mfma_slice(1);
-    IMEX_SCHED_SLICE();
-    read_frags(cur, 3, 1);
-    mfma_slice(0);
-    IMEX_SCHED_SLICE();
-    mfma_slice(1);
-    __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): this wavefront's copies have landed
-    __syncthreads();                    // ... and so have everyone else's
-    read_frags(cur ^ 1, 0, 0);
-  };
+  // prologue: tiles 0 .. kDist-1 in flight, tile 0 landed, its first fragments in registers
+#pragma unroll
+  for (int t = 0; t < kDist; ++t)
+    dma_tile(min(t, lastTile), t * kRStage);
+  wait_vmcnt<(kDist - 1) * (kRADma + kRBDma)>();
+  __builtin_amdgcn_s_barrier();
+  IMEX_FENCE();
+#pragma unroll
+  for (int i = 0; i < TI; ++i) read_a(0, 0, 0, i);
+#pragma unroll
+  for (int j = 0; j < TJ; ++j) read_b(0, 0, 0, j);
+  IMEX_FENCE();
 
-  dma_tile(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0f70);
-  __syncthreads();
-  read_frags(0, 0, 0);
-  int kt = 0;
-  for (; kt + 1 < kTiles; kt += 2) { // two steps per trip: the LDS stage is a compile-time constant
-    k_step(kt, Stage0{});
-    k_step(kt + 1, Stage1{});
+  int curOff = 0;                    // stage of tile t
+  int nxtOff = kRStage;              // stage of tile t+1
+  int dmaOff = kDist * kRStage;      // stage tile t+kDist goes to (= stage of tile t-1)
+  for (int t = 0; t < kTiles; ++t) {
+    // the stage of tile t-1 is free: every wavefront passed the previous step's barrier
+    // after its last reads of it
+    dma_tile(min(t + kDist, lastTile), dmaOff);
+    IMEX_FENCE();
+    slice(0, curOff, 1);             // multiplies k 0-15 of tile t, reads its k 16-31
+    wait_vmcnt<(kDist - 1) * (kRADma + kRBDma)>(); // tile t+1 has landed (this wavefront's part)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();    // ... and everyone else's; all reads of tile t are done
+    IMEX_FENCE();
+    slice(1, nxtOff, 0);             // multiplies k 16-31 of tile t, reads k 0-15 of tile t+1
+    curOff = nxtOff;
+    nxtOff = nxtOff + kRStage == kStages * kRStage ? 0 : nxtOff + kRStage;
+    dmaOff = dmaOff + kRStage == kStages * kRStage ? 0 : dmaOff + kRStage;
   }
-  if (kt < kTiles)
-    k_step(kt, Stage0{});
+  wait_vmcnt<0>();
 
-  // -- epilogue: lane holds, for tile (i,j), column n = lane%32 and rows
-  //    (r/4)*8 + (lane/32)*4 + r%4, r = 0..15.
 #pragma unroll
   for (int i = 0; i < TI; ++i)
 #pragma unroll
@@ -344,8 +310,8 @@ template <typename T, typename Epi>
 __device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
                                            Epi epi) {
   // 2 stages x (256 + 256) rows x 64 k x 2 B = 128 KiB of the CU's 160 KiB LDS.
-  __shared__ __attribute__((aligned(16))) char lds[2 * kStageBytes];
-  const bool tileable = (M % BM == 0) && (N % BN == 0) && (K % BK == 0) && M > 0 && N > 0 && K > 0 &&
+  __shared__ __attribute__((aligned(16))) char lds[kStages * kRStage];
+  const bool tileable = (M % BM == 0) && (N % BN == 0) && (K % RK == 0) && M > 0 && N > 0 && K > 0 &&
                         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
   if (tileable)
     gemm_tiled<T, Epi>(A, B, M, N, K, epi, lds);

@@ -162,7 +162,7 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
   }
   case Shape::Gemm: { // 512 lanes: eight wavefronts per 256 x 256 tile
     const int64_t M = dims[0], N = dims[1], K = dims[2];
-    const bool tileable = M > 0 && N > 0 && K > 0 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0;
+    const bool tileable = M > 0 && N > 0 && K > 0 && M % 256 == 0 && N % 256 == 0 && K % 32 == 0;
     block[0] = 512;
     grid[0] = tileable ? static_cast<size_t>((M / 256) * (N / 256)) : ceilDiv(M * N, 512);
     break;

@@ -240,7 +240,7 @@ def test_gemm_golden_3x3(host, orc, stream):
     assert np.all(orc.half_to_float(out) == g["expected_fill"])
 
 
-@pytest.mark.parametrize("M,N,K", [(5, 7, 9), (100, 36, 130), (256, 256, 32), (255, 256, 64), (17, 300, 64)])
+@pytest.mark.parametrize("M,N,K", [(5, 7, 9), (100, 36, 130), (256, 256, 16), (256, 256, 48), (255, 256, 64), (17, 300, 64)])
 def test_gemm_untileable_shapes_bit_exact(host, orc, stream, M, N, K):
     a = orc.fill_uniform(M * K, "f16", 1, -1, 1).reshape(M, K)
     b = orc.fill_uniform(K * N, "f16", 2, -1, 1).reshape(K, N)
@@ -264,7 +264,8 @@ def test_gemm_tiled_identity_and_layout(host, orc, stream, dtype):
     assert np.array_equal(got, np.outer(a1[:, 77], orc.to_float(b, dtype)[77]).astype(np.float32))
 
 
-@pytest.mark.parametrize("dtype,M,N,K", [("f16", 512, 768, 4096), ("bf16", 256, 1024, 1024), ("f16", 1024, 256, 64)])
+@pytest.mark.parametrize("dtype,M,N,K", [("f16", 512, 768, 4096), ("bf16", 256, 1024, 1024), ("f16", 1024, 256, 64),
+                                           ("f16", 256, 256, 32), ("bf16", 512, 256, 96), ("f16", 256, 512, 160)])
 def test_gemm_tiled_small_integers_exact(host, orc, stream, dtype, M, N, K):
     """|a|,|b| <= 4: every partial sum is an integer below 2^24, so any
     accumulation order gives the same f32 bits as the integer product."""
@@ -273,6 +274,33 @@ def test_gemm_tiled_small_integers_exact(host, orc, stream, dtype, M, N, K):
     want = orc.to_float(a, dtype).astype(np.int64) @ orc.to_float(b, dtype).astype(np.int64)
     got = host.gemm(stream, a, b, ab_dtype=dtype)
     assert np.array_equal(got.astype(np.int64), want)
+
+
+@pytest.mark.parametrize("dtype,M,N,K", [("f16", 256, 256, 32), ("bf16", 256, 512, 96), ("f16", 512, 256, 224)])
+def test_gemm_tiled_short_k_random(host, orc, stream, dtype, M, N, K):
+    """K shorter than the copy pipeline is deep (1, 3 and 7 steps of 32): the
+    prologue and the clamped tail copies must not disturb the result."""
+    a = orc.fill_uniform(M * K, dtype, 11, -1, 1).reshape(M, K)
+    b = orc.fill_uniform(K * N, dtype, 12, -1, 1).reshape(K, N)
+    assert gemm_close(host.gemm(stream, a, b, ab_dtype=dtype), orc.gemm(a, b, dtype))
+
+
+def test_gemm_launch_shape_slack(host, orc, stream):
+    """A grid with more workgroups than tiles (tiled path) or fewer threads than
+    outputs (one-thread-per-output path) still computes every element once."""
+    import ctypes as C
+    for (M, N, K, grid) in [(256, 256, 64, 9), (100, 36, 130, 2)]:
+        a = orc.fill_uniform(M * K, "f16", 21, -1, 1).reshape(M, K)
+        b = orc.fill_uniform(K * N, "f16", 22, -1, 1).reshape(K, N)
+        d_a, d_b, d_c = stream.to_device(a), stream.to_device(b), stream.alloc(M * N * 4)
+        fn = stream.kernel("imex_gemm_f16_f16_f32")
+        descs, keep = host._pack_params([d_a, d_b, d_c, M, N, K])
+        stream.rt.gpuLaunchKernel(stream.handle, fn, grid, 1, 1, 512, 1, 1, 0, C.cast(descs, C.c_void_p), None)
+        stream.wait()
+        got = stream.from_device(d_c, (M, N), np.float32)
+        assert gemm_close(got, orc.gemm(a, b, "f16"))
+        for p in (d_a, d_b, d_c):
+            stream.free(p)
 
 
 def test_gemm_config_f16_4096(host, orc, stream):

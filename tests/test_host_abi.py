@@ -75,6 +75,11 @@ def test_launch_shapes(host):
     assert ls("imex_gemm_f16_f16_f32", [4096, 4096, 4096]) == ((256, 1, 1), (512, 1, 1), 0)
     assert ls("imex_gemm_bf16_bias_silu_bf16", [4096, 11008, 4096])[0] == (16 * 43, 1, 1)
     assert ls("imex_gemm_f16_f16_f32", [3, 3, 3])[0] == (1, 1, 1)
+    # the tiled path takes K in steps of 32: the catalogue must count tiles exactly when the kernel tiles
+    assert ls("imex_gemm_f16_f16_f32", [256, 256, 32])[0] == (1, 1, 1)
+    assert ls("imex_gemm_f16_f16_f32", [512, 256, 96])[0] == (2, 1, 1)
+    assert ls("imex_gemm_f16_f16_f32", [256, 256, 48])[0] == (128, 1, 1)
+    assert ls("imex_gemm_f16_f16_f32", [255, 256, 64])[0] == (128, 1, 1)
     assert ls("imex_gemm_4kx4kx4k_f16_f16_f32", []) == ((16, 16, 1), (512, 1, 1), 0)
     with pytest.raises(ValueError):
         ls("imex_relu_f32", [1, 2])
