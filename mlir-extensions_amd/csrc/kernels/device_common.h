@@ -34,16 +34,11 @@ __device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
 }
 
 // Cache policy helpers.  MI355X has 256 MiB of Infinity Cache behind the L2s.
-// Pure streaming kernels (element-wise, softmax, row sums) use non-temporal
-// accesses always.  The transposes use ordinary loads/stores while the tensor
-// pair fits the Infinity Cache -- it then merges their 256-byte row segments,
-// which measured 35% faster -- and non-temporal accesses above that size, where
-// evicting (and writing back) never-reused lines only costs bandwidth.
-#ifndef IMEX_CACHE_RESIDENT_BYTES
-#define IMEX_CACHE_RESIDENT_BYTES (int64_t(256) << 20)
-#endif
-constexpr int64_t kCacheResidentBytes = IMEX_CACHE_RESIDENT_BYTES;
-
+// Every kernel here touches each byte once, so the streaming kernels and the
+// transposes use non-temporal accesses: measured on tensors that are not already
+// cache-resident (buffers rotated through 2 GiB, or after a cache flush), that is
+// the faster policy everywhere.  Ordinary accesses only win when one and the same
+// buffer pair, small enough for the Infinity Cache, is processed again and again.
 template <bool kStream> __device__ __forceinline__ u32x4 load128(const u32x4 *p) {
   if constexpr (kStream)
     return __builtin_nontemporal_load(p);
