@@ -30,11 +30,18 @@
  *   imex_gemm_f16_f16_f32[_acc], imex_gemm_bf16_bf16_f32[_acc], imex_gemm_f16_f16_f16
  *                                  (A, B, C, M:i64, N:i64, K:i64)
  *       WG/gemm_4kx4kx4k_f16_f16_f32.mlir:47-91          dims = {M, N, K}
+ *   imex_gemm_f16_f16_f32_tb       (A, Bt, C, M:i64, N:i64, K:i64)   B stored [N,K]: C = A.B^T
+ *       WG/gemm_4kx4kx4k_transpose_b.mlir:53-88          dims = {M, N, K}
+ *   imex_gemm_f16_f16_f32_ta       (At, B, C, M:i64, N:i64, K:i64)   A stored [K,M]: C = A^T.B
+ *       WG/gemm_4kx4kx4k_transpose_a.mlir:31-55          dims = {M, N, K}
  *   imex_gemm_bf16_bias_silu_bf16  (A, B, bias, out, M:i64, N:i64, K:i64)
  *       WG/gemm_4kx4kx4k_f16_f16_f32_bias.mlir:88-113 + silu_gpu.mlir.in:3-19
  *   imex_gemm_4kx4kx4k_f16_f16_f32       (A, B, C)        dims = {}
  *   imex_gemm_4kx4kx4k_f16_f16_f32_bias  (bias, C, A, B)  dims = {}
- *       the reference kernels' own signatures (WG/...f32.mlir:48, ...bias.mlir:78)
+ *   imex_gemm_4kx4kx4k_transpose_b       (A, Bt, C)       dims = {}   C += A.B^T
+ *   imex_gemm_4kx4kx4k_transpose_a       (At, B, C)       dims = {}   C += A^T.B
+ *       the reference kernels' own signatures (WG/...f32.mlir:48, ...bias.mlir:78,
+ *       ...transpose_b.mlir:53, ...transpose_a.mlir:31)
  */
 #ifndef IMEX_HIP_KERNELS_H
 #define IMEX_HIP_KERNELS_H

@@ -81,6 +81,12 @@ std::vector<Workload> workloads() {
       {"gemm_f16_4096", "imex_gemm_f16_f16_f32", {K4, K4, K4},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, false, 2.0 * K4 * K4 * K4, true},
+      {"gemm_f16_4096_transpose_b", "imex_gemm_f16_f16_f32_tb", {K4, K4, K4},
+       {{Elem::F16, {K4, K4}, true, -0.5f, 0.5f}, {Elem::F16, {K4, K4}, true, -0.5f, 0.5f}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, false, 2.0 * K4 * K4 * K4, true},
+      {"gemm_f16_4096_transpose_a", "imex_gemm_f16_f16_f32_ta", {K4, K4, K4},
+       {{Elem::F16, {K4, K4}, true, -0.5f, 0.5f}, {Elem::F16, {K4, K4}, true, -0.5f, 0.5f}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, false, 2.0 * K4 * K4 * K4, true},
       {"gemm_mlp_bf16_4096x11008x4096", "imex_gemm_bf16_bias_silu_bf16", {K4, 11008, K4},
        {{Elem::BF16, {K4, K4}, true, -1.7f, 1.7f}, {Elem::BF16, {K4, 11008}, true, -0.035f, 0.035f},
         {Elem::F32, {11008}, true, -0.17f, 0.17f}, {Elem::BF16, {K4, 11008}, false, 0, 0}},

@@ -55,11 +55,9 @@ constexpr int RK = 32;                              // K per step (one ring stag
 constexpr int WM = BM / kWavesM, WN = BN / kWavesN; // wavefront tile
 constexpr int TI = WM / 32, TJ = WN / 32;           // MFMA 32x32 tiles per wavefront
 constexpr int kStages = 4;                          // LDS ring: 4 x 32 KiB of the 160 KiB
-constexpr int kRA = BM * RK * 2;                    // A image [256 rows][32 k], 16-byte groups swizzled
-constexpr int kRB = RK * BN * 2;                    // B image [32 k][256 n], 32-byte pairs swizzled
-constexpr int kRStage = kRA + kRB;
-constexpr int kRADma = kRA / 1024 / kWaves;         // 1 KiB global->LDS copies per wavefront and step (A)
-constexpr int kRBDma = kRB / 1024 / kWaves;         // ... (B)
+constexpr int kImageBytes = 256 * RK * 2;           // one operand's 256 x 32 slab: 16 KiB
+constexpr int kRStage = 2 * kImageBytes;            // A image + B image
+constexpr int kDmaPerWave = kImageBytes / 1024 / kWaves; // 1 KiB global->LDS copies per wavefront, operand and step
 constexpr int kDist = kStages - 1;                  // tiles in flight ahead of the one being multiplied
 constexpr int kGroupM = 4;                          // tile rows per L2-sharing group
 
@@ -125,7 +123,9 @@ struct StoreF16 {       // C(f16) = acc   (WG/gemm_4kx4kx4k_f16_f16_f16.mlir)
 };
 
 // ---- one-thread-per-output path ---------------------------------------------------
-template <typename T, typename Epi>
+// kAT: A is stored [K,M] (A[k*M+m]) instead of [M,K]; kBT: B is stored [N,K]
+// (B[n*K+k]) instead of [K,N].
+template <typename T, bool kAT, bool kBT, typename Epi>
 __device__ __forceinline__ void gemm_scalar(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
                                             Epi epi) {
   // grid-stride, so that any launch shape covers every output
@@ -135,7 +135,9 @@ __device__ __forceinline__ void gemm_scalar(const uint16_t *A, const uint16_t *B
     const int64_t m = idx / N, n = idx % N;
     float acc = 0.0f;
     for (int64_t k = 0; k < K; ++k) {
-      const float p = T::widen(A[m * K + k]) * T::widen(B[k * N + n]);
+      const float a = T::widen(kAT ? A[k * M + m] : A[m * K + k]);
+      const float b = T::widen(kBT ? B[n * K + k] : B[k * N + n]);
+      const float p = a * b;
       acc = acc + p; // rounded multiply, rounded add (file is built with contraction off)
     }
     epi(m, n, N, acc);
@@ -150,13 +152,93 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, in
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, range, 0x00020000);
 }
 
-
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
   __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <typename T, typename Epi>
+// One MFMA operand of a workgroup tile: a 256 x 32 (rows x k) slab per step.  Both
+// A (rows = m) and B (rows = n) want, per lane, row = lane % 32 of a 32-row
+// fragment and the 8 consecutive k starting at (lane / 32) * 8.
+//
+// KContig: the slab is k-contiguous in memory (A as [M,K], B as [N,K]).  LDS image
+//   [256 rows][32 k], 64-byte rows; 16-byte group c of row r is stored at group
+//   c ^ ((r >> 2) & 3), which makes the 128-bit fragment reads conflict-free.  One
+//   1 KiB copy = 16 rows.  A fragment is one ds_read_b128.
+// KStrided: the slab's rows are strided in memory (B as [K,N], A as [K,M]).  LDS
+//   image [32 k][256 rows], 512-byte rows; 32-byte pair p of k-row r at pair
+//   p ^ g(r), g(r) = (r & 3) | ((r >> 3 & 1) << 2).  One copy = 2 k-rows.  A
+//   fragment is two LDS transpose reads (ds_read_b64_tr_b16): within each group of
+//   16 lanes, lane t supplies the address of 4 consecutive rows at k-row t/4 and
+//   receives 4 consecutive k of row t.
+// A direct global->LDS copy puts lane l's 16 bytes at base + 16 l, so the swizzle
+// is applied to the lane's GLOBAL address instead.
+template <typename T, bool kStrided, int kFrags> struct Operand {
+  __amdgpu_buffer_rsrc_t rsrc;
+  int voff[kDmaPerWave];         // per-lane byte offset of each copy at step 0
+  int step;                      // bytes per K-step in memory
+  int dstWave;                   // LDS byte offset of this wavefront's copies inside the image
+  int rd[kStrided ? kFrags : 2]; // per-lane LDS read bases: KStrided one per fragment, KContig one per slice
+
+  // ptr: the operand's matrix; ld: its leading dimension; first: first row (m0 or n0)
+  // of the slab; w0: the wavefront's first row inside the slab; extent: rows * cols.
+  __device__ __forceinline__ void setup(const uint16_t *ptr, int64_t ld, int64_t first, int w0, int64_t extent,
+                                        int wave, int lane) {
+    if constexpr (!kStrided) {
+      rsrc = make_rsrc(ptr + first * ld, 256 * ld * 2);
+#pragma unroll
+      for (int q = 0; q < kDmaPerWave; ++q) {
+        const int row = wave * (256 / kWaves) + q * 16 + (lane >> 2);
+        const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+        voff[q] = int((int64_t(row) * ld + chunk * 8) * 2);
+      }
+      step = RK * 2;
+      dstWave = wave * (256 / kWaves) * (RK * 2);
+      const int fragRow = lane & 31, fragHalf = lane >> 5;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+        rd[ks] = (w0 + fragRow) * (RK * 2) + ((((ks * 2 + fragHalf) ^ (fragRow >> 2)) & 3) << 4);
+    } else {
+      rsrc = make_rsrc(ptr + first, (extent - first) * 2);
+#pragma unroll
+      for (int q = 0; q < kDmaPerWave; ++q) {
+        const int row = wave * (RK / kWaves) + q * 2 + (lane >> 5);
+        const int g = (row & 3) | (((row >> 3) & 1) << 2);
+        const int chunk = (((((lane & 31) >> 1) ^ g)) << 1) | (lane & 1);
+        voff[q] = int((int64_t(row) * ld + chunk * 8) * 2);
+      }
+      step = int(RK * ld * 2);
+      dstWave = wave * (RK / kWaves) * 512;
+      const int t = lane & 15, block = (lane >> 4) & 1, khalf = lane >> 5;
+      const int g = (t >> 2) | (khalf << 2); // g(k-row) for k-row = ks*16 + khalf*8 + h*4 + t/4
+      const int pair0 = w0 / 16 + block;     // 32-byte pair holding this lane's rows, fragment 0
+#pragma unroll
+      for (int f = 0; f < kFrags; ++f)
+        rd[f] = (khalf * 8 + (t >> 2)) * 512 + (((pair0 + 2 * f) ^ g) * 32) + (t & 3) * 8;
+    }
+  }
+  // the wavefront's copies of K-step kt into the image at LDS byte offset `image`
+  __device__ __forceinline__ void dma(LdsChar *lds, int image, int kt) const {
+#pragma unroll
+    for (int q = 0; q < kDmaPerWave; ++q)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + image + dstWave + q * 1024, 16, voff[q], kt * step, 0, 0);
+  }
+  // fragment f (rows w0 + 32 f ...) of 16-wide slice ks of the image at `image`
+  __device__ __forceinline__ typename T::Frag read(const char *lds, int image, int ks, int f) const {
+    if constexpr (!kStrided) {
+      return *reinterpret_cast<const typename T::Frag *>(lds + image + rd[ks] + f * 32 * (RK * 2));
+    } else {
+      const char *p = lds + image + rd[f] + ks * 16 * 512;
+      const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p));           // k +0..3
+      const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p + 4 * 512)); // k +4..7
+      return __builtin_bit_cast(typename T::Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+  }
+};
+
+// kAT / kBT as in gemm_scalar.  A is KContig unless transposed; B is KContig only
+// when transposed.
+template <typename T, bool kAT, bool kBT, typename Epi>
 __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                            int64_t M, int64_t N, int64_t K, Epi epi, char *lds) {
   static_assert(TI == 4 && TJ == 2 && kWaves == 8, "written for 8 wavefronts of 4 x 2 MFMA tiles");
@@ -166,13 +248,14 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
   const int wave = tid >> 6;
   const int wm = wave / kWavesN, wn = wave % kWavesN;
 
+  // -- workgroup id -> tile, XCD-aware ------------------------------------------------
   const int tilesM = int(M / BM), tilesN = int(N / BN);
   const int tiles = tilesM * tilesN;
   int pid = blockIdx.y * gridDim.x + blockIdx.x;
   if (pid >= tiles)
     return; // a launch with more workgroups than tiles: the surplus has nothing to do
   if (tiles % 8 == 0)
-    pid = (pid % 8) * (tiles / 8) + pid / 8;
+    pid = (pid % 8) * (tiles / 8) + pid / 8; // ids congruent mod 8 share an XCD
   const int group = kGroupM * tilesN;
   const int firstM = (pid / group) * kGroupM;
   const int groupRows = min(tilesM - firstM, kGroupM);
@@ -180,52 +263,16 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
   const int tileN = (pid % group) / groupRows;
   const int64_t m0 = int64_t(tileM) * BM, n0 = int64_t(tileN) * BN;
 
-  // global -> LDS copies.  A image: 64-byte rows, 16-byte group c of row r stored at
-  // group c ^ ((r >> 2) & 3); one copy = 16 rows.  B image: 512-byte rows, 32-byte pair p
-  // of row r at pair p ^ g(r); one copy = 2 rows.
   const int waveU = __builtin_amdgcn_readfirstlane(wave);
-  const __amdgpu_buffer_rsrc_t aRsrc = make_rsrc(A + m0 * K, int64_t(BM) * K * 2);
-  const __amdgpu_buffer_rsrc_t bRsrc = make_rsrc(B + n0, (K * N - n0) * 2);
-  int aVoff[kRADma], bVoff[kRBDma];
-#pragma unroll
-  for (int q = 0; q < kRADma; ++q) {
-    const int row = wave * (BM / kWaves) + q * 16 + (lane >> 2);
-    const int chunk = (lane & 3) ^ ((row >> 2) & 3);
-    aVoff[q] = int((int64_t(row) * K + chunk * 8) * 2);
-  }
-#pragma unroll
-  for (int q = 0; q < kRBDma; ++q) {
-    const int row = wave * (RK / kWaves) + q * 2 + (lane >> 5);
-    const int g = (row & 3) | (((row >> 3) & 1) << 2);
-    const int chunk = (((((lane & 31) >> 1) ^ g)) << 1) | (lane & 1);
-    bVoff[q] = int((int64_t(row) * N + chunk * 8) * 2);
-  }
-  const int bStep = int(RK * N * 2);
-  auto dma_tile = [&](int kt, int stageOff) { // stageOff = byte offset of the stage, wave-uniform
-    LdsChar *aDst = lds_base + stageOff + waveU * (BM / kWaves) * (RK * 2);
-    LdsChar *bDst = lds_base + stageOff + kRA + waveU * (RK / kWaves) * 512;
-#pragma unroll
-    for (int q = 0; q < kRADma; ++q)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(aRsrc, aDst + q * 1024, 16, aVoff[q], kt * (RK * 2), 0, 0);
-#pragma unroll
-    for (int q = 0; q < kRBDma; ++q)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(bRsrc, bDst + q * 1024, 16, bVoff[q], kt * bStep, 0, 0);
+  Operand<T, kAT, TI> opA;
+  Operand<T, !kBT, TJ> opB;
+  opA.setup(A, kAT ? M : K, m0, wm * WM, M * K, waveU, lane);
+  opB.setup(B, kBT ? K : N, n0, wn * WN, K * N, waveU, lane);
+  constexpr int kImgA = 0, kImgB = kImageBytes;
+  auto dma_tile = [&](int kt, int stageOff) { // stageOff: byte offset of the ring stage, wave-uniform
+    opA.dma(lds_base, stageOff + kImgA, kt);
+    opB.dma(lds_base, stageOff + kImgB, kt);
   };
-
-  const int fragRow = lane & 31, fragHalf = lane >> 5;
-  int aRd[2];
-#pragma unroll
-  for (int ks = 0; ks < 2; ++ks)
-    aRd[ks] = (wm * WM + fragRow) * (RK * 2) + ((((ks * 2 + fragHalf) ^ (fragRow >> 2)) & 3) << 4);
-  int bRd[TJ];
-  {
-    const int t = lane & 15, nblock = (lane >> 4) & 1, khalf = lane >> 5;
-    const int g = (t >> 2) | (khalf << 2);
-    const int pair0 = (wn * WN) / 16 + nblock;
-#pragma unroll
-    for (int j = 0; j < TJ; ++j)
-      bRd[j] = kRA + (khalf * 8 + (t >> 2)) * 512 + (((pair0 + 2 * j) ^ g) * 32) + (t & 3) * 8;
-  }
 
   f32x16 acc[TI][TJ];
 #pragma unroll
@@ -237,17 +284,11 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
         acc[i][j][r] = 0.0f;
 
   typename T::Frag af[2][TI], bf[2][TJ];
-  auto read_a = [&](int stageOff, int ks, int buf, int i) {
-    af[buf][i] = *reinterpret_cast<const typename T::Frag *>(lds + stageOff + aRd[ks] + i * 32 * (RK * 2));
-  };
-  auto read_b = [&](int stageOff, int ks, int buf, int j) {
-    const char *p = lds + stageOff + bRd[j] + ks * 16 * 512;
-    const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p));
-    const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p + 4 * 512));
-    bf[buf][j] = __builtin_bit_cast(typename T::Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-  };
+  auto read_a = [&](int stageOff, int ks, int buf, int i) { af[buf][i] = opA.read(lds, stageOff + kImgA, ks, i); };
+  auto read_b = [&](int stageOff, int ks, int buf, int j) { bf[buf][j] = opB.read(lds, stageOff + kImgB, ks, j); };
   auto mm = [&](int buf, int i, int j) { acc[i][j] = T::mfma(af[buf][i], bf[buf][j], acc[i][j]); };
-  // 8 MFMAs from register buffer `buf`, interleaved with the 8 LDS reads that fill buf^1
+  // 8 MFMAs from register buffer `buf`, interleaved by hand with the LDS reads that
+  // fill buf^1 (the fences keep the compiler from regrouping them)
   auto slice = [&](int buf, int rOff, int rks) {
     mm(buf, 0, 0); read_a(rOff, rks, buf ^ 1, 0); IMEX_FENCE();
     mm(buf, 0, 1); read_a(rOff, rks, buf ^ 1, 1); IMEX_FENCE();
@@ -265,7 +306,7 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
 #pragma unroll
   for (int t = 0; t < kDist; ++t)
     dma_tile(min(t, lastTile), t * kRStage);
-  wait_vmcnt<(kDist - 1) * (kRADma + kRBDma)>();
+  wait_vmcnt<(kDist - 1) * 2 * kDmaPerWave>();
   __builtin_amdgcn_s_barrier();
   IMEX_FENCE();
 #pragma unroll
@@ -274,26 +315,30 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
   for (int j = 0; j < TJ; ++j) read_b(0, 0, 0, j);
   IMEX_FENCE();
 
-  int curOff = 0;                    // stage of tile t
-  int nxtOff = kRStage;              // stage of tile t+1
-  int dmaOff = kDist * kRStage;      // stage tile t+kDist goes to (= stage of tile t-1)
+  int curOff = 0;               // stage of tile t
+  int nxtOff = kRStage;         // stage of tile t+1
+  int dmaOff = kDist * kRStage; // stage tile t+kDist goes to (= stage of tile t-1)
   for (int t = 0; t < kTiles; ++t) {
-    // the stage of tile t-1 is free: every wavefront passed the previous step's barrier
-    // after its last reads of it
+    // The stage of tile t-1 is free: every wavefront passed the previous step's
+    // barrier after its last reads of it.  Past the end of K the copies re-fetch the
+    // last tile into a stage nobody reads, so every step is the same code.
     dma_tile(min(t + kDist, lastTile), dmaOff);
     IMEX_FENCE();
-    slice(0, curOff, 1);             // multiplies k 0-15 of tile t, reads its k 16-31
-    wait_vmcnt<(kDist - 1) * (kRADma + kRBDma)>(); // tile t+1 has landed (this wavefront's part)
+    slice(0, curOff, 1);                            // multiplies k 0-15 of tile t, reads its k 16-31
+    wait_vmcnt<(kDist - 1) * 2 * kDmaPerWave>();    // tile t+1 has landed (this wavefront's part) ...
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();    // ... and everyone else's; all reads of tile t are done
+    __builtin_amdgcn_s_barrier();                   // ... and everyone else's; all reads of tile t are done
     IMEX_FENCE();
-    slice(1, nxtOff, 0);             // multiplies k 16-31 of tile t, reads k 0-15 of tile t+1
+    slice(1, nxtOff, 0);                            // multiplies k 16-31 of tile t, reads k 0-15 of tile t+1
     curOff = nxtOff;
     nxtOff = nxtOff + kRStage == kStages * kRStage ? 0 : nxtOff + kRStage;
     dmaOff = dmaOff + kRStage == kStages * kRStage ? 0 : dmaOff + kRStage;
   }
   wait_vmcnt<0>();
 
+  // -- epilogue: lane holds, for tile (i,j), column n = lane%32 and rows
+  //    (r/4)*8 + (lane/32)*4 + r%4, r = 0..15.
+  const int fragRow = lane & 31, fragHalf = lane >> 5;
 #pragma unroll
   for (int i = 0; i < TI; ++i)
 #pragma unroll
@@ -306,17 +351,17 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
       }
 }
 
-template <typename T, typename Epi>
+template <typename T, bool kAT, bool kBT, typename Epi>
 __device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
                                            Epi epi) {
-  // 2 stages x (256 + 256) rows x 64 k x 2 B = 128 KiB of the CU's 160 KiB LDS.
+  // 4 stages x (256 + 256) rows x 32 k x 2 B = 128 KiB of the CU's 160 KiB LDS.
   __shared__ __attribute__((aligned(16))) char lds[kStages * kRStage];
   const bool tileable = (M % BM == 0) && (N % BN == 0) && (K % RK == 0) && M > 0 && N > 0 && K > 0 &&
                         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
   if (tileable)
-    gemm_tiled<T, Epi>(A, B, M, N, K, epi, lds);
+    gemm_tiled<T, kAT, kBT, Epi>(A, B, M, N, K, epi, lds);
   else
-    gemm_scalar<T, Epi>(A, B, M, N, K, epi);
+    gemm_scalar<T, kAT, kBT, Epi>(A, B, M, N, K, epi);
 }
 
 } // namespace
@@ -325,30 +370,30 @@ __device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B,
 extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_f16_f16_f32(const uint16_t *A, const uint16_t *B,
                                                                             float *C, int64_t M, int64_t N,
                                                                             int64_t K) {
-  gemm_entry<F16>(A, B, M, N, K, StoreF32{C});
+  gemm_entry<F16, false, false>(A, B, M, N, K, StoreF32{C});
 }
 // C += A.B
 extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_f16_f16_f32_acc(const uint16_t *A,
                                                                                 const uint16_t *B, float *C,
                                                                                 int64_t M, int64_t N, int64_t K) {
-  gemm_entry<F16>(A, B, M, N, K, AccumulateF32{C});
+  gemm_entry<F16, false, false>(A, B, M, N, K, AccumulateF32{C});
 }
 extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_bf16_bf16_f32(const uint16_t *A,
                                                                               const uint16_t *B, float *C,
                                                                               int64_t M, int64_t N, int64_t K) {
-  gemm_entry<BF16>(A, B, M, N, K, StoreF32{C});
+  gemm_entry<BF16, false, false>(A, B, M, N, K, StoreF32{C});
 }
 extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_bf16_bf16_f32_acc(const uint16_t *A,
                                                                                   const uint16_t *B, float *C,
                                                                                   int64_t M, int64_t N,
                                                                                   int64_t K) {
-  gemm_entry<BF16>(A, B, M, N, K, AccumulateF32{C});
+  gemm_entry<BF16, false, false>(A, B, M, N, K, AccumulateF32{C});
 }
 // C(f16) = A.B
 extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_f16_f16_f16(const uint16_t *A, const uint16_t *B,
                                                                             uint16_t *C, int64_t M, int64_t N,
                                                                             int64_t K) {
-  gemm_entry<F16>(A, B, M, N, K, StoreF16{C});
+  gemm_entry<F16, false, false>(A, B, M, N, K, StoreF16{C});
 }
 // out(bf16) = silu(A.B + bias[n])
 extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_bf16_bias_silu_bf16(const uint16_t *A,
@@ -356,7 +401,21 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_bf16_bias_silu_
                                                                                     const float *bias,
                                                                                     uint16_t *out, int64_t M,
                                                                                     int64_t N, int64_t K) {
-  gemm_entry<BF16>(A, B, M, N, K, BiasSiluBF16{out, bias});
+  gemm_entry<BF16, false, false>(A, B, M, N, K, BiasSiluBF16{out, bias});
+}
+
+// C = A . B^T with B stored [N,K] (WG/gemm_4kx4kx4k_transpose_b.mlir:16,70-83: the
+// B tile is loaded k-contiguous and transposed in registers before the dpas)
+extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_f16_f16_f32_tb(const uint16_t *A, const uint16_t *Bt,
+                                                                               float *C, int64_t M, int64_t N,
+                                                                               int64_t K) {
+  gemm_entry<F16, false, true>(A, Bt, M, N, K, StoreF32{C});
+}
+// C = A^T . B with A stored [K,M] (WG/gemm_4kx4kx4k_transpose_a.mlir:41-47)
+extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_f16_f16_f32_ta(const uint16_t *At, const uint16_t *B,
+                                                                               float *C, int64_t M, int64_t N,
+                                                                               int64_t K) {
+  gemm_entry<F16, true, false>(At, B, M, N, K, StoreF32{C});
 }
 
 // Fixed-shape entry points with the reference kernels' own signatures, so the
@@ -366,11 +425,23 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_bf16_bias_silu_
 extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_4kx4kx4k_f16_f16_f32(const uint16_t *A,
                                                                                      const uint16_t *B,
                                                                                      float *C) {
-  gemm_entry<F16>(A, B, 4096, 4096, 4096, AccumulateF32{C});
+  gemm_entry<F16, false, false>(A, B, 4096, 4096, 4096, AccumulateF32{C});
+}
+//   gemm_4kx4kx4k_transpose_b.mlir:40,53   args (A, B[N,K], C), C += A.B^T
+//   gemm_4kx4kx4k_transpose_a.mlir:21,31   args (A[K,M], B, C), C += A^T.B
+extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_4kx4kx4k_transpose_b(const uint16_t *A,
+                                                                                     const uint16_t *Bt,
+                                                                                     float *C) {
+  gemm_entry<F16, false, true>(A, Bt, 4096, 4096, 4096, AccumulateF32{C});
+}
+extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_4kx4kx4k_transpose_a(const uint16_t *At,
+                                                                                     const uint16_t *B,
+                                                                                     float *C) {
+  gemm_entry<F16, true, false>(At, B, 4096, 4096, 4096, AccumulateF32{C});
 }
 extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_4kx4kx4k_f16_f16_f32_bias(const float *bias,
                                                                                           float *C,
                                                                                           const uint16_t *A,
                                                                                           const uint16_t *B) {
-  gemm_entry<F16>(A, B, 4096, 4096, 4096, BiasAccumulateF32{C, bias});
+  gemm_entry<F16, false, false>(A, B, 4096, 4096, 4096, BiasAccumulateF32{C, bias});
 }

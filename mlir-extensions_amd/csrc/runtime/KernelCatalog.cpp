@@ -60,7 +60,13 @@ const Entry kEntries[] = {
     {"imex_gemm_f16_f16_f16", "(A: f16*, B: f16*, C: f16*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
     {"imex_gemm_bf16_bias_silu_bf16", "(A: bf16*, B: bf16*, bias: f32*, out: bf16*, M: i64, N: i64, K: i64)",
      Module::Gemm, Shape::Gemm, 3},
+    {"imex_gemm_f16_f16_f32_tb", "(A: f16*, Bt: f16* [N,K], C: f32*, M: i64, N: i64, K: i64)", Module::Gemm,
+     Shape::Gemm, 3},
+    {"imex_gemm_f16_f16_f32_ta", "(At: f16* [K,M], B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm,
+     Shape::Gemm, 3},
     {"imex_gemm_4kx4kx4k_f16_f16_f32", "(A: f16*, B: f16*, C: f32*)", Module::Gemm, Shape::GemmFixed4k, 0},
+    {"imex_gemm_4kx4kx4k_transpose_b", "(A: f16*, Bt: f16* [N,K], C: f32*)", Module::Gemm, Shape::GemmFixed4k, 0},
+    {"imex_gemm_4kx4kx4k_transpose_a", "(At: f16* [K,M], B: f16*, C: f32*)", Module::Gemm, Shape::GemmFixed4k, 0},
     {"imex_gemm_4kx4kx4k_f16_f16_f32_bias", "(bias: f32*, C: f32*, A: f16*, B: f16*)", Module::Gemm,
      Shape::GemmFixed4k, 0},
 };

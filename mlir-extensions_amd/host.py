@@ -375,15 +375,22 @@ def transpose3d(stream, x):
                   out_shape=(d2, d1, d0))
 
 
-def gemm(stream, a, b, c=None, ab_dtype="f16", out_dtype="f32"):
-    """C = A.B (or C += A.B when `c` is given), WG/gemm_4kx4kx4k_f16_f16_f32.mlir:21-91."""
+def gemm(stream, a, b, c=None, ab_dtype="f16", out_dtype="f32", trans_a=False, trans_b=False):
+    """C = A.B (or C += A.B when `c` is given), WG/gemm_4kx4kx4k_f16_f16_f32.mlir:21-91.
+    trans_a: `a` is stored [K,M] (WG/gemm_4kx4kx4k_transpose_a.mlir); trans_b: `b` is
+    stored [N,K] (WG/gemm_4kx4kx4k_transpose_b.mlir)."""
     _check(a, ab_dtype)
     _check(b, ab_dtype)
-    M, K = a.shape
-    K2, N = b.shape
+    K, M = a.shape if trans_a else a.shape[::-1]
+    K2, N = b.shape[::-1] if trans_b else b.shape
     if K != K2:
         raise ValueError("inner dimensions differ: %d vs %d" % (K, K2))
-    if out_dtype == "f16":
+    if trans_a or trans_b:
+        if (trans_a and trans_b) or c is not None or ab_dtype != "f16" or out_dtype != "f32":
+            raise ValueError("the transposed-operand kernels are f16 -> f32, one operand transposed, no accumulate")
+        name = "imex_gemm_f16_f16_f32_ta" if trans_a else "imex_gemm_f16_f16_f32_tb"
+        out_np = np.float32
+    elif out_dtype == "f16":
         name = "imex_gemm_f16_f16_f16"
         out_np = np.uint16
     else:
