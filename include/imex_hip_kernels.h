@@ -27,6 +27,11 @@
  *       benchmarks/transpose/transpose2d_gpu.mlir.in:4-11 dims = {rows, cols}
  *   imex_transpose3d_b16 / _b32    (in, out, d0:i64, d1:i64, d2:i64)
  *       benchmarks/transpose/transpose3d_gpu.mlir.in:4-11 dims = {d0, d1, d2}
+ *   imex_loop_fusion_f32 / _f16 / _bf16   (a, b, out, n:i64)         out = (log a + |b|) - a
+ *       benchmarks/kLoopFusion/kLoopFusion.mlir.in:4-30  dims = {n}
+ *   imex_input_fusion_f32 / _f16 / _bf16  (a, b, out, rows:i64, cols:i64)
+ *       out[j] = sum_i (log b[i,j] + |a[i,j]|)
+ *       benchmarks/kInputFusion/kInputFusion.mlir.in:6-40 dims = {rows, cols}
  *   imex_gemm_f16_f16_f32[_acc], imex_gemm_bf16_bf16_f32[_acc], imex_gemm_f16_f16_f16
  *                                  (A, B, C, M:i64, N:i64, K:i64)
  *       WG/gemm_4kx4kx4k_f16_f16_f32.mlir:47-91          dims = {M, N, K}

@@ -1,0 +1,223 @@
+// Fused element-wise chains of the reference's kLoopFusion / kInputFusion
+// benchmarks, each as ONE pass over HBM.
+//
+// Reference op bodies:
+//   benchmarks/kLoopFusion/kLoopFusion.mlir.in:4-30
+//       t1 = log(a); t2 = |b|; t3 = t1 + t2; out = t3 - a          (four generics,
+//       three full-size temporaries in the reference's lowering)
+//   benchmarks/kInputFusion/kInputFusion.mlir.in:6-40
+//       t = log(b) + |a|  (same first three generics, on swapped arguments), then
+//       out[j] = 0 + sum_i t[i][j]: a reduction over the ROWS, one output per
+//       column, added in ascending i (indexing maps (d1,d0) -> (d0), :29-39).
+//
+// Every operation is a separately rounded f32 one, as in the reference; log is
+// the host libm's logf (benchmarks/pipelines/linalg-to-cpu.pp:18-19 lowers
+// math.log to it), restated below so that the device lands on the same bits.
+// 16-bit variants widen to f32, run the same chain and round once at the end
+// (the policy the reference applies to 16-bit types on the GPU,
+// docs/Transforms/BF16ToGpu.md:17-26).
+//
+// Arguments:  loop fusion  (a, b, out, n: i64)              dims = {n}
+//             input fusion (a, b, out, rows: i64, cols: i64) dims = {rows, cols}
+// Launch: block (256,1,1); loop fusion grid ceil(n / 4096) (f32) or ceil(n / 8192)
+// (16-bit); input fusion grid ceil(cols / 256), one thread per output column.
+
+#include "device_common.h"
+
+using namespace imexhip;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kVecsPerThread = 4;
+
+// ---------------------------------------------------------------------------
+// logf as glibc computes it (Arm Optimized Routines logf: x = 2^k z with z in
+// [0x3f330000, ...), c = table centre of z's 1/16 sub-interval, r = z/c - 1,
+// log x = k ln2 + log c + r + r^2 (A2 + A1 r + A0 r^2); all in f64 with IEEE
+// operations, one final rounding).  A host build of this function agrees with
+// libm's logf on every positive finite f32.
+// ---------------------------------------------------------------------------
+struct LogfEntry {
+  double invc, logc;
+};
+__device__ const LogfEntry kLogfTable[16] = {
+    {0x1.661ec79f8f3bep+0, -0x1.57bf7808caadep-2}, {0x1.571ed4aaf883dp+0, -0x1.2bef0a7c06ddbp-2},
+    {0x1.49539f0f010bp+0, -0x1.01eae7f513a67p-2},  {0x1.3c995b0b80385p+0, -0x1.b31d8a68224e9p-3},
+    {0x1.30d190c8864a5p+0, -0x1.6574f0ac07758p-3}, {0x1.25e227b0b8eap+0, -0x1.1aa2bc79c81p-3},
+    {0x1.1bb4a4a1a343fp+0, -0x1.a4e76ce8c0e5ep-4}, {0x1.12358f08ae5bap+0, -0x1.1973c5a611cccp-4},
+    {0x1.0953f419900a7p+0, -0x1.252f438e10c1ep-5}, {0x1p+0, 0x0p+0},
+    {0x1.e608cfd9a47acp-1, 0x1.aa5aa5df25984p-5},  {0x1.ca4b31f026aap-1, 0x1.c5e53aa362eb4p-4},
+    {0x1.b2036576afce6p-1, 0x1.526e57720db08p-3},  {0x1.9c2d163a1aa2dp-1, 0x1.bc2860d22477p-3},
+    {0x1.886e6037841edp-1, 0x1.1058bc8a07ee1p-2},  {0x1.767dcf5534862p-1, 0x1.4043057b6ee09p-2},
+};
+
+__device__ __forceinline__ float logf_libm(float x, const LogfEntry *table) {
+  uint32_t ix = f2u(x);
+  if (ix == 0x3f800000u)
+    return 0.0f;
+  if (ix - 0x00800000u >= 0x7f800000u - 0x00800000u) {
+    if (ix * 2 == 0)
+      return -__builtin_inff(); // log(+-0)
+    if (ix == 0x7f800000u)
+      return x;                 // log(inf)
+    if ((ix & 0x80000000u) || ix * 2 >= 0xff000000u)
+      return __builtin_nanf(""); // negative or NaN
+    ix = f2u(x * 0x1p23f);      // subnormal: normalise
+    ix -= 23u << 23;
+  }
+  const uint32_t tmp = ix - 0x3f330000u;
+  const int i = (tmp >> 19) & 15;
+  const int k = static_cast<int32_t>(tmp) >> 23;
+  const uint32_t iz = ix - (tmp & 0xff800000u);
+  const double invc = table[i].invc, logc = table[i].logc;
+  const double z = static_cast<double>(u2f(iz));
+  const double r = z * invc - 1.0;
+  const double y0 = logc + static_cast<double>(k) * 0x1.62e42fefa39efp-1;
+  const double r2 = r * r;
+  double y = 0x1.5575b0be00b6ap-2 * r + -0x1.ffffef20a4123p-2;
+  y = -0x1.00ea348b88334p-2 * r2 + y;
+  y = y * r2 + (y0 + r);
+  return static_cast<float>(y);
+}
+
+__device__ __forceinline__ void stage_table(LogfEntry *lds) {
+  if (threadIdx.x < 16)
+    lds[threadIdx.x] = kLogfTable[threadIdx.x];
+  __syncthreads();
+}
+
+// the chains, on f32 values
+__device__ __forceinline__ float loop_chain(float a, float b, const LogfEntry *table) {
+  const float t1 = logf_libm(a, table);
+  const float t2 = __builtin_fabsf(b);
+  const float t3 = t1 + t2;
+  return t3 - a;
+}
+__device__ __forceinline__ float input_chain(float a, float b, const LogfEntry *table) {
+  const float t1 = logf_libm(b, table);
+  const float t2 = __builtin_fabsf(a);
+  return t1 + t2;
+}
+
+enum class Dt { F32, F16, BF16 };
+template <Dt D> struct Elem;
+template <> struct Elem<Dt::F32> {
+  static constexpr int kBytes = 4, kPerVec = 4;
+  static __device__ __forceinline__ float get(const void *p, int64_t i) { return static_cast<const float *>(p)[i]; }
+  static __device__ __forceinline__ void put(void *p, int64_t i, float v) { static_cast<float *>(p)[i] = v; }
+  static __device__ __forceinline__ void unpack(u32x4 v, float *f) {
+    f[0] = u2f(v.x); f[1] = u2f(v.y); f[2] = u2f(v.z); f[3] = u2f(v.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float *f) { return u32x4{f2u(f[0]), f2u(f[1]), f2u(f[2]), f2u(f[3])}; }
+};
+template <bool kBf> struct Elem16 {
+  static constexpr int kBytes = 2, kPerVec = 8;
+  static __device__ __forceinline__ float widen(uint32_t h) { return kBf ? bf16_bits_to_float(h) : half_bits_to_float(h); }
+  static __device__ __forceinline__ uint32_t narrow(float f) { return kBf ? float_to_bf16_bits(f) : float_to_half_bits(f); }
+  static __device__ __forceinline__ float get(const void *p, int64_t i) { return widen(static_cast<const uint16_t *>(p)[i]); }
+  static __device__ __forceinline__ void put(void *p, int64_t i, float v) {
+    static_cast<uint16_t *>(p)[i] = static_cast<uint16_t>(narrow(v));
+  }
+  static __device__ __forceinline__ void unpack(u32x4 v, float *f) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = widen(w[i] & 0xffffu);
+      f[2 * i + 1] = widen(w[i] >> 16);
+    }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float *f) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      w[i] = narrow(f[2 * i]) | (narrow(f[2 * i + 1]) << 16);
+    return u32x4{w[0], w[1], w[2], w[3]};
+  }
+};
+template <> struct Elem<Dt::F16> : Elem16<false> {};
+template <> struct Elem<Dt::BF16> : Elem16<true> {};
+
+// ---- kLoopFusion: two streams in, one out ------------------------------------------
+template <Dt D>
+__device__ __forceinline__ void loop_fusion(const void *__restrict__ a, const void *__restrict__ b,
+                                            void *__restrict__ out, int64_t n) {
+  using E = Elem<D>;
+  __shared__ LogfEntry table[16];
+  stage_table(table);
+  constexpr int64_t kElemsPerBlock = int64_t(kThreads) * kVecsPerThread * E::kPerVec;
+  const int64_t base = int64_t(blockIdx.x) * kElemsPerBlock;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+                         reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  if (aligned && base + kElemsPerBlock <= n) {
+    const u32x4 *pa = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a) + base * E::kBytes);
+    const u32x4 *pb = reinterpret_cast<const u32x4 *>(static_cast<const char *>(b) + base * E::kBytes);
+    u32x4 *po = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + base * E::kBytes);
+    u32x4 va[kVecsPerThread], vb[kVecsPerThread];
+#pragma unroll
+    for (int j = 0; j < kVecsPerThread; ++j) {
+      va[j] = load128<true>(pa + j * kThreads + threadIdx.x);
+      vb[j] = load128<true>(pb + j * kThreads + threadIdx.x);
+    }
+#pragma unroll
+    for (int j = 0; j < kVecsPerThread; ++j) {
+      float fa[E::kPerVec], fb[E::kPerVec];
+      E::unpack(va[j], fa);
+      E::unpack(vb[j], fb);
+#pragma unroll
+      for (int i = 0; i < E::kPerVec; ++i)
+        fa[i] = loop_chain(fa[i], fb[i], table);
+      store128<true>(E::pack(fa), po + j * kThreads + threadIdx.x);
+    }
+  } else {
+    for (int64_t i = base + threadIdx.x; i < base + kElemsPerBlock && i < n; i += kThreads)
+      E::put(out, i, loop_chain(E::get(a, i), E::get(b, i), table));
+  }
+}
+
+// ---- kInputFusion: chain + column sums ------------------------------------------------
+// One thread per output column, rows added in ascending order from +0.0 -- the
+// reference's order, so the f32 result is the same bits.  Consecutive lanes read
+// consecutive columns (coalesced); eight rows of loads are in flight per lane.
+template <Dt D>
+__device__ __forceinline__ void input_fusion(const void *__restrict__ a, const void *__restrict__ b,
+                                             void *__restrict__ out, int64_t rows, int64_t cols) {
+  using E = Elem<D>;
+  __shared__ LogfEntry table[16];
+  stage_table(table);
+  const int64_t stride = int64_t(gridDim.x) * kThreads;
+  for (int64_t col = int64_t(blockIdx.x) * kThreads + threadIdx.x; col < cols; col += stride) {
+    float acc = 0.0f;
+    int64_t i = 0;
+    for (; i + 8 <= rows; i += 8) {
+      float xa[8], xb[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        xa[u] = E::get(a, (i + u) * cols + col);
+        xb[u] = E::get(b, (i + u) * cols + col);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        acc = acc + input_chain(xa[u], xb[u], table);
+    }
+    for (; i < rows; ++i)
+      acc = acc + input_chain(E::get(a, i * cols + col), E::get(b, i * cols + col), table);
+    E::put(out, col, acc);
+  }
+}
+
+} // namespace
+
+#define IMEX_FUSION_KERNELS(SUFFIX, DT, CTYPE)                                                                       \
+  extern "C" __global__ __launch_bounds__(kThreads) void imex_loop_fusion_##SUFFIX(                                  \
+      const CTYPE *a, const CTYPE *b, CTYPE *out, int64_t n) {                                                       \
+    loop_fusion<DT>(a, b, out, n);                                                                                   \
+  }                                                                                                                  \
+  extern "C" __global__ __launch_bounds__(kThreads) void imex_input_fusion_##SUFFIX(                                 \
+      const CTYPE *a, const CTYPE *b, CTYPE *out, int64_t rows, int64_t cols) {                                      \
+    input_fusion<DT>(a, b, out, rows, cols);                                                                         \
+  }
+
+IMEX_FUSION_KERNELS(f32, Dt::F32, float)
+IMEX_FUSION_KERNELS(f16, Dt::F16, uint16_t)
+IMEX_FUSION_KERNELS(bf16, Dt::BF16, uint16_t)

@@ -20,12 +20,13 @@ extern const unsigned char imex_blob_softmax[], imex_blob_softmax_end[];
 extern const unsigned char imex_blob_reduce[], imex_blob_reduce_end[];
 extern const unsigned char imex_blob_transpose[], imex_blob_transpose_end[];
 extern const unsigned char imex_blob_gemm[], imex_blob_gemm_end[];
+extern const unsigned char imex_blob_fusion[], imex_blob_fusion_end[];
 }
 
 namespace {
 
-enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm };
-enum class Shape { Eltwise32, Eltwise16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmFixed4k };
+enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm, Fusion };
+enum class Shape { Eltwise32, Eltwise16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmFixed4k, ColumnThreads };
 
 struct Entry {
   const char *name;
@@ -52,6 +53,15 @@ const Entry kEntries[] = {
      Shape::Transpose3D32, 3},
     {"imex_transpose3d_b16", "(in: b16*, out: b16*, d0: i64, d1: i64, d2: i64)", Module::Transpose,
      Shape::Transpose3D16, 3},
+    {"imex_loop_fusion_f32", "(a: f32*, b: f32*, out: f32*, n: i64)", Module::Fusion, Shape::Eltwise32, 1},
+    {"imex_loop_fusion_f16", "(a: f16*, b: f16*, out: f16*, n: i64)", Module::Fusion, Shape::Eltwise16, 1},
+    {"imex_loop_fusion_bf16", "(a: bf16*, b: bf16*, out: bf16*, n: i64)", Module::Fusion, Shape::Eltwise16, 1},
+    {"imex_input_fusion_f32", "(a: f32*, b: f32*, out: f32*, rows: i64, cols: i64)", Module::Fusion,
+     Shape::ColumnThreads, 2},
+    {"imex_input_fusion_f16", "(a: f16*, b: f16*, out: f16*, rows: i64, cols: i64)", Module::Fusion,
+     Shape::ColumnThreads, 2},
+    {"imex_input_fusion_bf16", "(a: bf16*, b: bf16*, out: bf16*, rows: i64, cols: i64)", Module::Fusion,
+     Shape::ColumnThreads, 2},
     {"imex_gemm_f16_f16_f32", "(A: f16*, B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
     {"imex_gemm_f16_f16_f32_acc", "(A: f16*, B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
     {"imex_gemm_bf16_bf16_f32", "(A: bf16*, B: bf16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
@@ -106,6 +116,7 @@ extern "C" const void *imexHipKernelModule(const char *kernel, size_t *size) {
   case Module::Reduce: begin = imex_blob_reduce; end = imex_blob_reduce_end; break;
   case Module::Transpose: begin = imex_blob_transpose; end = imex_blob_transpose_end; break;
   case Module::Gemm: begin = imex_blob_gemm; end = imex_blob_gemm_end; break;
+  case Module::Fusion: begin = imex_blob_fusion; end = imex_blob_fusion_end; break;
   }
   if (size)
     *size = static_cast<size_t>(end - begin);
@@ -166,6 +177,9 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     grid[2] = static_cast<size_t>(dims[1]);
     break;
   }
+  case Shape::ColumnThreads: // one lane per output column
+    grid[0] = ceilDiv(dims[1], 256);
+    break;
   case Shape::Gemm: { // 512 lanes: eight wavefronts per 256 x 256 tile
     const int64_t M = dims[0], N = dims[1], K = dims[2];
     const bool tileable = M > 0 && N > 0 && K > 0 && M % 256 == 0 && N % 256 == 0 && K % 32 == 0;

@@ -339,6 +339,34 @@ def silu(stream, x):
     return _unary(stream, "imex_silu_f32", x, "f32", [x.size])
 
 
+def _binary(stream, kernel, a, b, dtype, dims, out_shape):
+    _check(a, dtype)
+    _check(b, dtype)
+    if a.shape != b.shape:
+        raise ValueError("operand shapes differ: %s vs %s" % (a.shape, b.shape))
+    n_out = int(np.prod(out_shape))
+    d_a, d_b = stream.to_device(a), stream.to_device(b)
+    d_out = stream.alloc(max(n_out, 1) * a.dtype.itemsize)
+    try:
+        stream.launch(kernel, dims, [d_a, d_b, d_out] + list(dims))
+        stream.wait()
+        return stream.from_device(d_out, out_shape, a.dtype)
+    finally:
+        for p in (d_a, d_b, d_out):
+            stream.free(p)
+
+
+def loop_fusion(stream, a, b, dtype="f32"):
+    """benchmarks/kLoopFusion/kLoopFusion.mlir.in:4-30: (log a + |b|) - a"""
+    return _binary(stream, "imex_loop_fusion_" + dtype, a, b, dtype, [a.size], a.shape)
+
+
+def input_fusion(stream, a, b, dtype="f32"):
+    """benchmarks/kInputFusion/kInputFusion.mlir.in:6-40: out[j] = sum_i (log b[i,j] + |a[i,j]|)"""
+    rows, cols = a.shape
+    return _binary(stream, "imex_input_fusion_" + dtype, a, b, dtype, [rows, cols], (cols,))
+
+
 def softmax(stream, x, dtype="f32"):
     """benchmarks/softmax/softmax_gpu.mlir.in:4-44 (last dim of a 2-D tensor)"""
     rows, cols = x.shape

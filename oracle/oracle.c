@@ -242,6 +242,37 @@ void oracle_silu_f32(const float *x, float *y, size_t n) {
   for (size_t i = 0; i < n; ++i) y[i] = oracle_silu_scalar_f32(x[i]);
 }
 
+/* benchmarks/kLoopFusion/kLoopFusion.mlir.in:6-29: log, absf, addf, subf -- four
+   separately rounded f32 ops; log is libm logf on the CPU path. */
+void oracle_loop_fusion_f32(const float *a, const float *b, float *out, size_t n) {
+  for (size_t i = 0; i < n; ++i) {
+    float t1 = logf(a[i]);
+    float t2 = fabsf(b[i]);
+    float t3 = t1 + t2;
+    out[i] = t3 - a[i];
+  }
+}
+
+/* benchmarks/kInputFusion/kInputFusion.mlir.in:8-39: log of the SECOND argument,
+   absf of the first, addf, then out[j] = 0 + sum over rows i (ascending) of
+   t[i][j] (maps (d1,d0) -> (d0), d1 the reduction). */
+void oracle_input_fusion_f32(const float *a, const float *b, float *out, int64_t rows, int64_t cols) {
+  for (int64_t j = 0; j < cols; ++j) {
+    float acc = 0.0f;
+    for (int64_t i = 0; i < rows; ++i) {
+      float t1 = logf(b[i * cols + j]);
+      float t2 = fabsf(a[i * cols + j]);
+      float t3 = t1 + t2;
+      acc = acc + t3;
+    }
+    out[j] = acc;
+  }
+}
+
+void oracle_logf_n(const float *in, float *out, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = logf(in[i]);
+}
+
 float oracle_expf_cr(float x) { return (float)exp((double)x); }
 
 void oracle_expf_n(const float *in, float *out, size_t n) {

@@ -22,8 +22,11 @@
  *       the compiler's _Float16 / numpy; NaN payload behaviour parity unpinned;
  *   silu                                          : parity unpinned by reference
  *       tests (the reference holds no SiLU vector); pinned by closed forms only;
- *   expf                                          : host libm, as the reference's
- *       CPU lowering calls it; parity unpinned beyond 1 ulp.
+ *   expf, logf                                    : host libm, as the reference's
+ *       CPU lowering calls it; parity unpinned beyond 1 ulp;
+ *   loop fusion / input fusion chains             : parity unpinned by reference
+ *       tests (the benchmarks feed constants and check nothing); pinned by closed
+ *       forms against an f64 evaluation.
  */
 #ifndef IMEX_ORACLE_H
 #define IMEX_ORACLE_H
@@ -62,6 +65,9 @@ void oracle_relu_16(const uint16_t *x, uint16_t *y, size_t n, int dtype);
 void oracle_relu_olt_f32(const float *x, float *y, size_t n);          /* test/PlaidML/OpTest.Relu.mlir:29-35 */
 void oracle_silu_f32(const float *x, float *y, size_t n);              /* benchmarks/silu/silu_gpu.mlir.in:8-18 */
 float oracle_silu_scalar_f32(float x);
+void oracle_loop_fusion_f32(const float *a, const float *b, float *out, size_t n);                    /* benchmarks/kLoopFusion/kLoopFusion.mlir.in:6-29 */
+void oracle_input_fusion_f32(const float *a, const float *b, float *out, int64_t rows, int64_t cols); /* benchmarks/kInputFusion/kInputFusion.mlir.in:8-39 */
+void oracle_logf_n(const float *in, float *out, size_t n);              /* the host libm logf the fused chains call */
 float oracle_expf_cr(float x);                                          /* correctly rounded exp via f64 */
 void oracle_expf_n(const float *in, float *out, size_t n);              /* the host libm expf the oracle's silu/softmax call */
 

@@ -169,6 +169,27 @@ def silu_f32(x):
     return y
 
 
+def loop_fusion_f32(a, b):
+    a, b = _c(a, np.float32), _c(b, np.float32)
+    out = np.empty_like(a)
+    lib().oracle_loop_fusion_f32(_p(a), _p(b), _p(out), C.c_size_t(a.size))
+    return out
+
+
+def input_fusion_f32(a, b):
+    a, b = _c(a, np.float32), _c(b, np.float32)
+    out = np.empty(a.shape[1], np.float32)
+    lib().oracle_input_fusion_f32(_p(a), _p(b), _p(out), C.c_int64(a.shape[0]), C.c_int64(a.shape[1]))
+    return out
+
+
+def logf(x):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().oracle_logf_n(_p(x), _p(out), C.c_size_t(x.size))
+    return out
+
+
 def softmax_f32(x, three_pass=False):
     x = _c(x, np.float32)
     y = np.empty_like(x)

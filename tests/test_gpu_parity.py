@@ -218,6 +218,64 @@ def test_transpose3d(host, orc, stream, shape):
     assert np.array_equal(host.transpose3d(stream, x16), x16.transpose(2, 1, 0))
 
 
+# ========================= fused element-wise chains ========================
+@pytest.mark.parametrize("shape", [(512, 1024), (7, 13), (1, 4097), (300, 1000)])
+def test_loop_fusion_f32_bit_exact(host, orc, stream, shape):
+    """kLoopFusion: the device logf is the host libm's algorithm, every op is a
+    separately rounded f32 one, so the result is the oracle's bit for bit."""
+    n = int(np.prod(shape))
+    a = orc.fill_uniform(n, "f32", 41, 0.01, 40.0).reshape(shape)
+    b = orc.fill_uniform(n, "f32", 42, -5.0, 5.0).reshape(shape)
+    a.flat[:6] = [3.3, 1.0, 1e-40, 0.0, np.inf, 0.99999994]
+    got = host.loop_fusion(stream, a, b)
+    want = orc.loop_fusion_f32(a, b)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_loop_fusion_logf_sweep(host, orc, stream):
+    """b = 0 and exact cancellation aside, out + a = log a: sweep log over 16M bit
+    patterns of the whole positive range through the fused kernel."""
+    bits = (np.arange(1 << 24, dtype=np.uint64) * 127 + 1).astype(np.uint32) % np.uint32(0x7f800000)
+    a = bits.view(np.float32)
+    b = np.zeros_like(a)
+    got = host.loop_fusion(stream, a, b)
+    want = orc.loop_fusion_f32(a, b)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_loop_fusion_16bit(host, orc, stream, dtype):
+    n = 512 * 1024 + 77
+    a = orc.fill_uniform(n, dtype, 43, 0.05, 30.0)
+    b = orc.fill_uniform(n, dtype, 44, -5.0, 5.0)
+    got = orc.to_float(host.loop_fusion(stream, a, b, dtype), dtype)
+    # widen, f32 chain, one rounding at the end
+    want = orc.to_float(orc.from_float(orc.loop_fusion_f32(orc.to_float(a, dtype), orc.to_float(b, dtype)), dtype), dtype)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("shape", [(512, 1024), (9, 5), (1000, 300), (3, 2049)])
+def test_input_fusion_f32_bit_exact(host, orc, stream, shape):
+    """kInputFusion: column sums in row order from +0.0, as the reference adds them."""
+    n = int(np.prod(shape))
+    a = orc.fill_uniform(n, "f32", 45, -5.0, 5.0).reshape(shape)
+    b = orc.fill_uniform(n, "f32", 46, 0.01, 40.0).reshape(shape)
+    got = host.input_fusion(stream, a, b)
+    want = orc.input_fusion_f32(a, b)
+    assert got.shape == (shape[1],)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_input_fusion_16bit(host, orc, stream, dtype):
+    rows, cols = 512, 1024
+    a = orc.fill_uniform(rows * cols, dtype, 47, -2.0, 2.0).reshape(rows, cols)
+    b = orc.fill_uniform(rows * cols, dtype, 48, 0.5, 4.0).reshape(rows, cols)
+    got = orc.to_float(host.input_fusion(stream, a, b, dtype), dtype)
+    want = orc.to_float(orc.from_float(orc.input_fusion_f32(orc.to_float(a, dtype), orc.to_float(b, dtype)), dtype), dtype)
+    assert np.array_equal(got, want)
+
+
 # =============================== GEMM ======================================
 def gemm_close(got, ref):
     return np.max(np.abs(got - ref)) <= 5e-3 * np.max(np.abs(ref))

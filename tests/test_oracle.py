@@ -161,6 +161,60 @@ def test_libm_expf_vs_correctly_rounded(orc):
     assert got[0] == np.float32(math.exp(float(x[0]))) or ulps[0] == 1
 
 
+# ---- fused element-wise chains ------------------------------------------------------
+def test_libm_logf_vs_correctly_rounded(orc):
+    """The host libm logf the fused chains call is within 1 ulp of the correctly
+    rounded logarithm over the positive range, subnormals included."""
+    bits = np.concatenate([np.random.default_rng(7).integers(1, 0x7f800000, 400000, dtype=np.uint32),
+                           np.array([1, 2, 0x007fffff, 0x00800000, 0x3f800000, 0x3f7fffff, 0x3f800001, 0x7f7fffff],
+                                    np.uint32)])
+    x = bits.view(np.float32)
+    got = orc.logf(x)
+    cr = np.log(x.astype(np.float64)).astype(np.float32)
+    assert np.max(orc.ulp_distance_f32(got, cr)) <= 1
+    special = orc.logf(np.array([0.0, -0.0, np.inf, -1.0, np.nan], np.float32))
+    assert special[0] == -np.inf and special[1] == -np.inf and special[2] == np.inf
+    assert np.isnan(special[3]) and np.isnan(special[4])
+
+
+def test_fused_chains_closed_forms(orc):
+    """No vector for these chains exists in the reference (its benchmarks feed the
+    constants 3.3 and 1.0 and check nothing): the oracle is held against an f64
+    evaluation, the benchmark's own constants, and the argument roles."""
+    rng = np.random.default_rng(11)
+    a = rng.uniform(0.05, 50.0, (37, 53)).astype(np.float32)
+    b = rng.uniform(-9.0, 9.0, (37, 53)).astype(np.float32)
+    got = orc.loop_fusion_f32(a, b).astype(np.float64)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    exact = (np.log(a64) + np.abs(b64)) - a64
+    # three roundings of quantities no larger than max(|log a| + |b|, a) ~ 60
+    assert np.max(np.abs(got - exact)) <= 3 * 60 * 2.0 ** -24
+    # benchmark constants: (log 3.3 + |1.0|) - 3.3, op by op in f32
+    t1 = np.float32(math.log(3.3000000953674316))  # logf is correctly rounded here (checked above to 1 ulp)
+    want = np.float32(np.float32(t1 + np.float32(1.0)) - np.float32(3.3))
+    one = orc.loop_fusion_f32(np.full(4, 3.3, np.float32), np.full(4, 1.0, np.float32))
+    assert np.all(np.abs(one - want) <= np.spacing(np.float32(1.2)))
+    # log applies to the FIRST argument, abs to the second: swapping them changes the result
+    assert orc.loop_fusion_f32(np.float32([2.0]), np.float32([-8.0]))[0] == np.float32(np.float32(math.log(2.0)) + 8.0) - np.float32(2.0)
+    # input fusion: log of the SECOND argument, abs of the first, column sums in row order
+    col = orc.input_fusion_f32(b, a).astype(np.float64)   # a > 0 goes under the log
+    exact_col = (np.log(a64) + np.abs(b64)).sum(axis=0)
+    assert col.shape == (53,)
+    assert np.max(np.abs(col - exact_col)) <= 37 * 2 * 400 * 2.0 ** -24
+    # order of the adds: row order, starting from +0.0 (reproduced with numpy f32 scalars)
+    t = (orc.logf(a) + np.abs(b)).astype(np.float32)
+    acc = np.zeros(53, np.float32)
+    for i in range(37):
+        acc = (acc + t[i]).astype(np.float32)
+    assert np.array_equal(orc.input_fusion_f32(b, a), acc)
+    # benchmark constants: 512 rows of (log 1.0 + |3.3|) = 512 * 3.3f exactly representable sums? compare to the loop
+    c = orc.input_fusion_f32(np.full((512, 8), 3.3, np.float32), np.full((512, 8), 1.0, np.float32))
+    acc = np.float32(0.0)
+    for _ in range(512):
+        acc = np.float32(acc + np.float32(3.3))
+    assert np.all(c == acc)
+
+
 # ---- softmax ---------------------------------------------------------------------
 @pytest.mark.parametrize("key", ["softmax_f32_10x20", "softmax_f32_10x20_spirv"])
 def test_softmax_golden(orc, key):
