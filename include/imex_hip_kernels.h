@@ -32,6 +32,9 @@
  *   imex_input_fusion_f32 / _f16 / _bf16  (a, b, out, rows:i64, cols:i64)
  *       out[j] = sum_i (log b[i,j] + |a[i,j]|)
  *       benchmarks/kInputFusion/kInputFusion.mlir.in:6-40 dims = {rows, cols}
+ *   imex_flash_attention_fwd_f16   (Q, K, V, Out, sm_scale:f32, ZH:i64, N_CTX:i64)
+ *       softmax(sm_scale Q K^T) V per (batch, head), head dim 64, tensors [(ZH*N_CTX), 64]
+ *       WG/flash_attention_fwd.mlir:25-307               dims = {ZH, N_CTX}
  *   imex_gemm_f16_f16_f32[_acc], imex_gemm_bf16_bf16_f32[_acc], imex_gemm_f16_f16_f16
  *                                  (A, B, C, M:i64, N:i64, K:i64)
  *       WG/gemm_4kx4kx4k_f16_f16_f32.mlir:47-91          dims = {M, N, K}

@@ -52,7 +52,7 @@ struct Workload {
   std::vector<int64_t> dims;    // what imexHipKernelLaunchShape takes
   std::vector<Tensor> tensors;  // kernel pointer arguments, in order
   std::vector<int64_t> indexArgs; // i64 arguments after the pointers
-  bool hasInit;                 // trailing f32 `init` argument (reductions)
+  int floatArg;                 // 0 none; 1 trailing f32 `init` (reductions); 2 f32 between pointers and indices (sm_scale)
   double work;                  // algorithmic bytes or flops per launch
   bool mfma;                    // roofline: MFMA (TFLOP/s) or HBM (GB/s)
 };
@@ -61,36 +61,42 @@ std::vector<Workload> workloads() {
   const int64_t K4 = 4096, K8 = 8192;
   return {
       {"relu_f32_4096x4096", "imex_relu_f32", {K4 * K4},
-       {{Elem::F32, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}}, {K4 * K4}, false,
+       {{Elem::F32, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}}, {K4 * K4}, 0,
        2.0 * K4 * K4 * 4, false},
       {"silu_f32_512x640x20x15", "imex_silu_f32", {98304000},
-       {{Elem::F32, {98304000}, true, -8, 8}, {Elem::F32, {98304000}, false, 0, 0}}, {98304000}, false,
+       {{Elem::F32, {98304000}, true, -8, 8}, {Elem::F32, {98304000}, 0, 0, 0}}, {98304000}, 0,
        2.0 * 98304000 * 4, false},
       {"softmax_f16_16384x1024", "imex_softmax_f16", {16384, 1024},
-       {{Elem::F16, {16384, 1024}, true, -4, 4}, {Elem::F16, {16384, 1024}, false, 0, 0}}, {16384, 1024}, false,
+       {{Elem::F16, {16384, 1024}, true, -4, 4}, {Elem::F16, {16384, 1024}, 0, 0, 0}}, {16384, 1024}, 0,
        2.0 * 16384 * 1024 * 2, false},
       {"rowsum_f32_8192x8192", "imex_rowsum_f32", {K8, K8},
-       {{Elem::F32, {K8, K8}, true, 0, 1}, {Elem::F32, {K8}, false, 0, 0}}, {K8, K8}, true,
+       {{Elem::F32, {K8, K8}, 1, 0, 1}, {Elem::F32, {K8}, false, 0, 0}}, {K8, K8}, 1,
        K8 * K8 * 4.0 + K8 * 4.0, false},
       {"transpose_bf16_8192x8192", "imex_transpose2d_b16", {K8, K8},
-       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, false,
+       {{Elem::BF16, {K8, K8}, 1, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, 0,
        2.0 * K8 * K8 * 2, false},
       {"transpose_f32_4096x4096", "imex_transpose2d_b32", {K4, K4},
-       {{Elem::F32, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}}, {K4, K4}, false,
+       {{Elem::F32, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}}, {K4, K4}, 0,
        2.0 * K4 * K4 * 4, false},
       {"gemm_f16_4096", "imex_gemm_f16_f16_f32", {K4, K4, K4},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
-       {K4, K4, K4}, false, 2.0 * K4 * K4 * K4, true},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true},
       {"gemm_f16_4096_transpose_b", "imex_gemm_f16_f16_f32_tb", {K4, K4, K4},
        {{Elem::F16, {K4, K4}, true, -0.5f, 0.5f}, {Elem::F16, {K4, K4}, true, -0.5f, 0.5f}, {Elem::F32, {K4, K4}, false, 0, 0}},
-       {K4, K4, K4}, false, 2.0 * K4 * K4 * K4, true},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true},
       {"gemm_f16_4096_transpose_a", "imex_gemm_f16_f16_f32_ta", {K4, K4, K4},
        {{Elem::F16, {K4, K4}, true, -0.5f, 0.5f}, {Elem::F16, {K4, K4}, true, -0.5f, 0.5f}, {Elem::F32, {K4, K4}, false, 0, 0}},
-       {K4, K4, K4}, false, 2.0 * K4 * K4 * K4, true},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true},
       {"gemm_mlp_bf16_4096x11008x4096", "imex_gemm_bf16_bias_silu_bf16", {K4, 11008, K4},
        {{Elem::BF16, {K4, K4}, true, -1.7f, 1.7f}, {Elem::BF16, {K4, 11008}, true, -0.035f, 0.035f},
         {Elem::F32, {11008}, true, -0.17f, 0.17f}, {Elem::BF16, {K4, 11008}, false, 0, 0}},
-       {K4, 11008, K4}, false, 2.0 * K4 * 11008 * K4, true},
+       {K4, 11008, K4}, 0, 2.0 * K4 * 11008 * K4, true},
+      // flash attention forward, the reference's shape: Z = 2, H = 2, N_CTX = 4096, D = 64, scale 0.5;
+      // 4 Z H N^2 D FLOP (two products)
+      {"flash_attention_f16_2x2x4096x64", "imex_flash_attention_fwd_f16", {4, K4},
+       {{Elem::F16, {4 * K4, 64}, true, -1, 1}, {Elem::F16, {4 * K4, 64}, true, -1, 1},
+        {Elem::F16, {4 * K4, 64}, true, -1, 1}, {Elem::F16, {4 * K4, 64}, false, 0, 0}},
+       {4, K4}, 2, 4.0 * 4 * K4 * K4 * 64, true},
   };
 }
 
@@ -147,13 +153,15 @@ int runWorkload(const Workload &w, const Options &opt) {
 
   // ParamDesc list: pointers, then i64 scalars, then the optional f32 init; {NULL,0} ends it.
   std::vector<int64_t> idx(w.indexArgs);
-  float init = 0.0f;
+  float init = 0.0f, scale = 0.5f;
   std::vector<ImexParamDesc> params;
   for (void *&p : dev)
     params.push_back({&p, sizeof(void *)});
+  if (w.floatArg == 2)
+    params.push_back({&scale, sizeof(float)});
   for (int64_t &v : idx)
     params.push_back({&v, sizeof(int64_t)});
-  if (w.hasInit)
+  if (w.floatArg == 1)
     params.push_back({&init, sizeof(float)});
   params.push_back({nullptr, 0});
   ImexEventDesc noDeps[1] = {{nullptr}};

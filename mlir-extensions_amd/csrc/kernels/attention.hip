@@ -1,0 +1,301 @@
+// Flash-attention forward, f16 in / f16 out, head dimension 64, no mask.
+//
+// Reference: test/Integration/Dialect/XeGPU/WG/flash_attention_fwd.mlir
+//   kernel :25-307 -- per workgroup a 128 x 64 Q tile, K/V walked in 64-key
+//   blocks, online softmax (running max m, running sum l, accumulator rescaled by
+//   exp(m_old - m_new)), P truncated to f16 before P.V, O = acc / l at the end;
+//   CPU check :332-421 -- softmax(scale * Q K^T) V per (batch, head), Q/K/V/O stored
+//   as [(Z*H*N_CTX), 64] row-major.
+//
+// On MI355X the products are formed TRANSPOSED, so that a lane owns one query:
+//   S^T[key, q] = K_tile . Q^T     A operand = K rows (k-contiguous in LDS),
+//                                  B operand = Q rows, loaded once into registers;
+//   O^T[d, q]  += V_tile^T . P^T   A operand = V^T via the LDS transpose read,
+//                                  B operand = P^T straight from the S^T
+//                                  accumulator registers (no shuffles: the MFMA's
+//                                  k index is bound to the keys in the order the
+//                                  accumulator holds them, and V^T is read in
+//                                  the same order).
+// With v_mfma_f32_32x32x16_f16 a lane holds query q = lane % 32 and, per 32-key
+// block, keys (r/4)*8 + (lane/32)*4 + r%4: the softmax max and sum over keys are
+// plain register loops plus ONE exchange between lane l and l+32 per block of
+// keys.
+//
+// Workgroup = 64 queries of one (batch, head): 4 wavefronts = 2 query halves x 2
+// key parities (wavefront w takes queries 32*(w&1).. and every second 64-key
+// tile, parity w>>1), partial (m, l, O) of the two parities merged through LDS at
+// the end.  That keeps 256 workgroups in flight for the reference's shape
+// (2 x 2 x 4096 x 64: one per CU) where a 128-query tile would fill half the
+// chip.  K and V tiles of 128 keys (both parities) go from global memory straight
+// into a three-stage LDS ring (buffer_load ... lds), two iterations ahead.
+//
+// Arguments: (Q, K, V, Out, sm_scale: f32, ZH: i64, N_CTX: i64)   dims = {ZH, N_CTX}
+//   ZH = batch * heads; N_CTX a multiple of 128; all four tensors [(ZH*N_CTX), 64].
+// Launch: block (256,1,1); grid (N_CTX/64, ZH, 1).  Other shapes take the
+// one-query-per-lane reference loop of the same kernel (grid-stride, any grid).
+
+#include "device_common.h"
+
+using namespace imexhip;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int D = 64;                 // head dimension
+constexpr int BM = 64;                // queries per workgroup
+constexpr int BN = 64;                // keys per tile; a ring stage holds two tiles (one per parity)
+constexpr int kTileBytes = BN * D * 2;          // 8 KiB
+constexpr int kStageBytes = 4 * kTileBytes;     // K0, K1, V0, V1 = 32 KiB
+constexpr int kStages = 3;
+constexpr int kDmaPerWave = kStageBytes / 1024 / 4; // 8 copies of 1 KiB per wavefront and stage
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) i16x4 LdsI16x4;
+typedef __attribute__((address_space(3))) char LdsChar;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, int64_t bytes) {
+  const int range = bytes > 0x7fffffff ? 0x7fffffff : int(bytes);
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, range, 0x00020000);
+}
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+// the value lane l+32 (or l-32) holds
+__device__ __forceinline__ float other_half(float v) { return __shfl_xor(v, 32, 64); }
+
+// ---- any-shape path: one lane per query, the reference loop ----------------------------
+__device__ __forceinline__ void attention_scalar(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                 uint16_t *Out, float scale, int64_t ZH, int64_t N) {
+  const int64_t block = int64_t(blockIdx.z) * gridDim.y * gridDim.x + int64_t(blockIdx.y) * gridDim.x + blockIdx.x;
+  const int64_t stride = int64_t(gridDim.x) * gridDim.y * gridDim.z * kThreads;
+  const float c = scale * 1.44269504088896341f;
+  for (int64_t row = block * kThreads + threadIdx.x; row < ZH * N; row += stride) {
+    const int64_t head0 = (row / N) * N;
+    float q[D], o[D];
+    for (int d = 0; d < D; ++d) {
+      q[d] = half_bits_to_float(Q[row * D + d]);
+      o[d] = 0.0f;
+    }
+    float m = -__builtin_inff(), l = 0.0f;
+    for (int64_t j = 0; j < N; ++j) {
+      float s = 0.0f;
+      for (int d = 0; d < D; ++d)
+        s += q[d] * half_bits_to_float(K[(head0 + j) * D + d]);
+      s *= c;
+      const float mNew = fmaxf(m, s);
+      const float alpha = exp2f(m - mNew);
+      const float p = half_bits_to_float(float_to_half_bits(exp2f(s - mNew)));
+      l = l * alpha + p;
+      for (int d = 0; d < D; ++d)
+        o[d] = o[d] * alpha + p * half_bits_to_float(V[(head0 + j) * D + d]);
+      m = mNew;
+    }
+    for (int d = 0; d < D; ++d)
+      Out[row * D + d] = static_cast<uint16_t>(float_to_half_bits(o[d] / l));
+  }
+}
+
+// ---- MFMA path ---------------------------------------------------------------------------
+__device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K,
+                                                const uint16_t *__restrict__ V, uint16_t *__restrict__ Out,
+                                                float scale, int64_t N, char *lds) {
+  LdsChar *ldsBase = (LdsChar *)lds;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wq = wave & 1, wk = wave >> 1;
+  const int qi = lane & 31, half = lane >> 5;
+  const int64_t head0 = int64_t(blockIdx.y) * N;         // first row of this (batch, head)
+  const int64_t q0 = head0 + int64_t(blockIdx.x) * BM + wq * 32;
+
+  // Q^T operand: lane (q, half) keeps Q[q][ds*16 + half*8 .. +7] for the four 16-wide steps
+  f16x8 qf[4];
+#pragma unroll
+  for (int ds = 0; ds < 4; ++ds)
+    qf[ds] = *reinterpret_cast<const f16x8 *>(Q + (q0 + qi) * D + ds * 16 + half * 8);
+
+  // -- global -> LDS copies.  A stage is [K tile 0][K tile 1][V tile 0][V tile 1], each 64
+  // rows of 128 bytes; one copy = 8 rows.  16-byte chunk c of row r is stored at
+  //   K: c ^ ((r ^ (r>>3 & 3)) & 7)   (conflict-free 128-bit fragment reads; same for r and r+32)
+  //   V: c ^ (((r>>1) & 1) << 2)     (conflict-free transpose reads)
+  // applied on the global side, since a direct copy fixes the lane's LDS position.
+  const __amdgpu_buffer_rsrc_t kRsrc = make_rsrc(K + head0 * D, N * D * 2);
+  const __amdgpu_buffer_rsrc_t vRsrc = make_rsrc(V + head0 * D, N * D * 2);
+  int kVoff[4], vVoff[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    // wavefront w copies rows [32w, 32w+32) of the stage's 128 K rows and of its 128 V rows
+    const int row = wave * 32 + c * 8 + (lane >> 3); // 0..127: key within the 128-key stage
+    const int r = row & 63;                          // row within its tile
+    const int kc = (lane & 7) ^ ((r ^ ((r >> 3) & 3)) & 7);
+    const int vc = (lane & 7) ^ (((r >> 1) & 1) << 2);
+    kVoff[c] = (row * D + kc * 8) * 2;
+    vVoff[c] = (row * D + vc * 8) * 2;
+  }
+  auto dma_stage = [&](int it, int stageOff) { // keys [128 it, 128 it + 128)
+    LdsChar *dst = ldsBase + stageOff + wave * 4096;
+    const int soff = it * (2 * BN * D * 2);
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kRsrc, dst + c * 1024, 16, kVoff[c], soff, 0, 0);
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vRsrc, dst + 2 * kTileBytes + c * 1024, 16, vVoff[c], soff, 0, 0);
+  };
+
+  // -- LDS read addresses (relative to this wavefront's K / V tile of a stage)
+  // K fragment (key block kb, step ds): row kb*32 + qi, logical chunk ds*2 + half
+  int kRd[4];
+#pragma unroll
+  for (int ds = 0; ds < 4; ++ds) {
+    const int r = qi; // the swizzle term is the same for rows r and r + 32
+    kRd[ds] = wk * kTileBytes + r * 128 + ((((ds * 2 + half) ^ r ^ ((r >> 3) & 3)) & 7) << 4);
+  }
+  // V^T fragment (d block db, key step kk): two transpose reads.  Lane t of a 16-lane group
+  // supplies the address of 4 consecutive d at key row (base + t/4) and receives 4 consecutive
+  // key rows of d = t.  Key rows of element e of the operand: kk*16 + (e/4)*8 + half*4 + e%4 --
+  // the order in which the S^T accumulator holds the keys.
+  int vRd[2];
+  {
+    const int t = lane & 15, blk = (lane >> 4) & 1;
+    const int row = half * 4 + (t >> 2);
+#pragma unroll
+    for (int db = 0; db < 2; ++db) {
+      const int chunk = ((db ^ ((t >> 3) & 1)) << 2) | (blk << 1) | ((t & 3) >> 1);
+      vRd[db] = 2 * kTileBytes + wk * kTileBytes + row * 128 + chunk * 16 + (t & 1) * 8;
+    }
+  }
+
+  f32x16 o[2];
+#pragma unroll
+  for (int db = 0; db < 2; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      o[db][r] = 0.0f;
+  float m = -__builtin_inff(); // running max of scale*log2(e)*s over this lane's query (both halves agree)
+  float l = 0.0f;              // running sum of p over THIS lane's keys only
+  const float c = scale * 1.44269504088896341f;
+
+  const int iters = int(N / (2 * BN));
+  dma_stage(0, 0);
+  dma_stage(min(1, iters - 1), kStageBytes);
+  int curOff = 0, dmaOff = 2 * kStageBytes;
+  for (int it = 0; it < iters; ++it) {
+    wait_vmcnt<kDmaPerWave>(); // stage `it` has landed (this wavefront's copies); the next one may be in flight
+    __builtin_amdgcn_s_barrier(); // ... everyone's; and everyone is done reading stage it-1
+    __builtin_amdgcn_sched_barrier(0);
+    dma_stage(min(it + 2, iters - 1), dmaOff); // into the stage read in iteration it-1
+    const char *st = lds + curOff;
+
+    // S^T = K . Q^T for this wavefront's 64 keys
+    f32x16 s[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        s[kb][r] = 0.0f;
+#pragma unroll
+      for (int ds = 0; ds < 4; ++ds) {
+        const f16x8 kf = *reinterpret_cast<const f16x8 *>(st + kRd[ds] + kb * 32 * 128);
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ds], s[kb], 0, 0, 0);
+      }
+    }
+    // online softmax over the keys; this lane owns 32 of the query's 64 scores
+    float mx = s[0][0];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        mx = fmaxf(mx, s[kb][r]);
+    mx = fmaxf(mx, other_half(mx));
+    const float mNew = fmaxf(m, mx * c);
+    const float alpha = __builtin_amdgcn_exp2f(m - mNew);
+    m = mNew;
+    float sum = 0.0f;
+    f16x8 pf[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __builtin_amdgcn_exp2f(s[kk >> 1][(kk & 1) * 8 + e] * c - mNew);
+        pf[kk][e] = static_cast<_Float16>(p); // the reference truncates P to f16 before P.V (:262-265)
+        sum += p;                             // ... and sums the untruncated f32 values (:243-247)
+      }
+    }
+    l = l * alpha + sum;
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        o[db][r] *= alpha;
+    // O^T += V^T . P^T
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+#pragma unroll
+      for (int db = 0; db < 2; ++db) {
+        const char *p = st + vRd[db] + kk * 16 * 128;
+        const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p));
+        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p + 8 * 128));
+        const f16x8 vf = __builtin_bit_cast(f16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[kk], o[db], 0, 0, 0);
+      }
+    }
+    curOff = curOff + kStageBytes == kStages * kStageBytes ? 0 : curOff + kStageBytes;
+    dmaOff = dmaOff + kStageBytes == kStages * kStageBytes ? 0 : dmaOff + kStageBytes;
+  }
+  wait_vmcnt<0>();
+  l += other_half(l); // both key halves of the lane pair
+
+  // -- merge the two key parities through LDS: wavefronts 2,3 hand (m, l, O^T) to 0,1
+  __syncthreads(); // the ring is free
+  float *xchg = reinterpret_cast<float *>(lds) + wq * (64 * 34);
+  if (wk == 1) {
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        xchg[(db * 16 + r) * 64 + lane] = o[db][r];
+    xchg[32 * 64 + lane] = m;
+    xchg[33 * 64 + lane] = l;
+  }
+  __syncthreads();
+  if (wk == 0) {
+    const float m1 = xchg[32 * 64 + lane], l1 = xchg[33 * 64 + lane];
+    const float mAll = fmaxf(m, m1);
+    const float a0 = exp2f(m - mAll), a1 = exp2f(m1 - mAll);
+    const float inv = 1.0f / (l * a0 + l1 * a1);
+    // lane holds, for query q = qi, d = db*32 + (r/4)*8 + half*4 + r%4
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f16x4 out4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = g * 4 + e;
+          out4[e] = static_cast<_Float16>((o[db][r] * a0 + xchg[(db * 16 + r) * 64 + lane] * a1) * inv);
+        }
+        *reinterpret_cast<f16x4 *>(Out + (q0 + qi) * D + db * 32 + g * 8 + half * 4) = out4;
+      }
+  }
+}
+
+} // namespace
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_flash_attention_fwd_f16(const uint16_t *Q,
+                                                                                   const uint16_t *K,
+                                                                                   const uint16_t *V,
+                                                                                   uint16_t *Out, float sm_scale,
+                                                                                   int64_t ZH, int64_t N_CTX) {
+  __shared__ __attribute__((aligned(16))) char lds[kStages * kStageBytes];
+  const bool tileable = N_CTX > 0 && N_CTX % (2 * BN) == 0 && gridDim.x == N_CTX / BM && gridDim.y == ZH &&
+                        gridDim.z == 1 &&
+                        ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
+                          reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(Out)) & 15) == 0;
+  if (tileable)
+    attention_tiled(Q, K, V, Out, sm_scale, N_CTX, lds);
+  else
+    attention_scalar(Q, K, V, Out, sm_scale, ZH, N_CTX);
+}

@@ -21,12 +21,13 @@ extern const unsigned char imex_blob_reduce[], imex_blob_reduce_end[];
 extern const unsigned char imex_blob_transpose[], imex_blob_transpose_end[];
 extern const unsigned char imex_blob_gemm[], imex_blob_gemm_end[];
 extern const unsigned char imex_blob_fusion[], imex_blob_fusion_end[];
+extern const unsigned char imex_blob_attention[], imex_blob_attention_end[];
 }
 
 namespace {
 
-enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm, Fusion };
-enum class Shape { Eltwise32, Eltwise16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmFixed4k, ColumnThreads };
+enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm, Fusion, Attention };
+enum class Shape { Eltwise32, Eltwise16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmFixed4k, ColumnThreads, Attention };
 
 struct Entry {
   const char *name;
@@ -62,6 +63,9 @@ const Entry kEntries[] = {
      Shape::ColumnThreads, 2},
     {"imex_input_fusion_bf16", "(a: bf16*, b: bf16*, out: bf16*, rows: i64, cols: i64)", Module::Fusion,
      Shape::ColumnThreads, 2},
+    {"imex_flash_attention_fwd_f16",
+     "(Q: f16*, K: f16*, V: f16*, Out: f16*, sm_scale: f32, ZH: i64, N_CTX: i64)", Module::Attention,
+     Shape::Attention, 2},
     {"imex_gemm_f16_f16_f32", "(A: f16*, B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
     {"imex_gemm_f16_f16_f32_acc", "(A: f16*, B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
     {"imex_gemm_bf16_bf16_f32", "(A: bf16*, B: bf16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
@@ -117,6 +121,7 @@ extern "C" const void *imexHipKernelModule(const char *kernel, size_t *size) {
   case Module::Transpose: begin = imex_blob_transpose; end = imex_blob_transpose_end; break;
   case Module::Gemm: begin = imex_blob_gemm; end = imex_blob_gemm_end; break;
   case Module::Fusion: begin = imex_blob_fusion; end = imex_blob_fusion_end; break;
+  case Module::Attention: begin = imex_blob_attention; end = imex_blob_attention_end; break;
   }
   if (size)
     *size = static_cast<size_t>(end - begin);
@@ -175,6 +180,16 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     grid[0] = ceilDiv(dims[2], tile);
     grid[1] = ceilDiv(dims[0], tile);
     grid[2] = static_cast<size_t>(dims[1]);
+    break;
+  }
+  case Shape::Attention: { // dims = {ZH, N_CTX}; 64 queries per workgroup when N_CTX % 128 == 0
+    const int64_t ZH = dims[0], N = dims[1];
+    if (N > 0 && N % 128 == 0 && ZH > 0 && ZH <= 65535) {
+      grid[0] = static_cast<size_t>(N / 64);
+      grid[1] = static_cast<size_t>(ZH);
+    } else {
+      grid[0] = ceilDiv(ZH * N, 256); // one lane per query
+    }
     break;
   }
   case Shape::ColumnThreads: // one lane per output column

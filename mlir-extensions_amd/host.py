@@ -367,6 +367,24 @@ def input_fusion(stream, a, b, dtype="f32"):
     return _binary(stream, "imex_input_fusion_" + dtype, a, b, dtype, [rows, cols], (cols,))
 
 
+def flash_attention(stream, q, k, v, zh, n_ctx, sm_scale):
+    """WG/flash_attention_fwd.mlir:25-307: softmax(sm_scale * Q K^T) V per (batch, head);
+    q, k, v f16 bit patterns [(zh * n_ctx), 64]."""
+    for t in (q, k, v):
+        _check(t, "f16")
+        if t.shape != (zh * n_ctx, 64):
+            raise ValueError("expected shape (%d, 64), got %s" % (zh * n_ctx, t.shape))
+    d_q, d_k, d_v = stream.to_device(q), stream.to_device(k), stream.to_device(v)
+    d_o = stream.alloc(max(q.size, 1) * 2)
+    try:
+        stream.launch("imex_flash_attention_fwd_f16", [zh, n_ctx], [d_q, d_k, d_v, d_o, float(sm_scale), zh, n_ctx])
+        stream.wait()
+        return stream.from_device(d_o, q.shape, np.uint16)
+    finally:
+        for p in (d_q, d_k, d_v, d_o):
+            stream.free(p)
+
+
 def softmax(stream, x, dtype="f32"):
     """benchmarks/softmax/softmax_gpu.mlir.in:4-44 (last dim of a 2-D tensor)"""
     rows, cols = x.shape

@@ -269,6 +269,51 @@ void oracle_input_fusion_f32(const float *a, const float *b, float *out, int64_t
   }
 }
 
+/* test/Integration/Dialect/XeGPU/WG/flash_attention_fwd.mlir:332-421 (cpu_impl):
+   per (batch, head), qk[i][j] = (sum_d q*k, f32, ascending d) * sm_scale; row max from
+   -inf; exp2((qk - max) * log2e); sequential row sum; divide; P truncated to f16;
+   out = f16(sum_k P[i][k] * v[k][j], f32, ascending k).  Q, K, V, out are
+   [(ZH * n_ctx), d_head] f16; only the listed rows (global row indices) are
+   computed, into out_rows[nrows][d_head]. */
+void oracle_flash_attention_rows(const uint16_t *Q, const uint16_t *K, const uint16_t *V, uint16_t *out_rows,
+                                 int64_t n_ctx, int64_t d_head, float sm_scale, const int64_t *rows,
+                                 int64_t nrows) {
+  const float log2e = 1.442695040888963f;
+  float *qk = (float *)malloc((size_t)n_ctx * sizeof(float));
+  for (int64_t ri = 0; ri < nrows; ++ri) {
+    const int64_t row = rows[ri];
+    const int64_t x_offset = (row / n_ctx) * n_ctx;
+    for (int64_t j = 0; j < n_ctx; ++j) {
+      float acc = 0.0f;
+      for (int64_t k = 0; k < d_head; ++k) {
+        float t = oracle_half_to_float(Q[row * d_head + k]) * oracle_half_to_float(K[(x_offset + j) * d_head + k]);
+        acc = acc + t;
+      }
+      qk[j] = acc * sm_scale;
+    }
+    float mx = -INFINITY;
+    for (int64_t j = 0; j < n_ctx; ++j) mx = (qk[j] > mx || mx != mx) ? qk[j] : mx; /* maximumf on non-NaN data */
+    for (int64_t j = 0; j < n_ctx; ++j) {
+      float t = qk[j] - mx;
+      float t1 = t * log2e;
+      qk[j] = exp2f(t1);
+    }
+    float sum = 0.0f;
+    for (int64_t j = 0; j < n_ctx; ++j) sum = sum + qk[j];
+    for (int64_t j = 0; j < n_ctx; ++j) qk[j] = qk[j] / sum;
+    for (int64_t j = 0; j < d_head; ++j) {
+      float pv = 0.0f;
+      for (int64_t k = 0; k < n_ctx; ++k) {
+        float p = oracle_half_to_float(oracle_float_to_half(qk[k]));
+        float t = p * oracle_half_to_float(V[(x_offset + k) * d_head + j]);
+        pv = t + pv;
+      }
+      out_rows[ri * d_head + j] = oracle_float_to_half(pv);
+    }
+  }
+  free(qk);
+}
+
 void oracle_logf_n(const float *in, float *out, size_t n) {
   for (size_t i = 0; i < n; ++i) out[i] = logf(in[i]);
 }

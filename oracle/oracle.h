@@ -24,6 +24,9 @@
  *       tests (the reference holds no SiLU vector); pinned by closed forms only;
  *   expf, logf                                    : host libm, as the reference's
  *       CPU lowering calls it; parity unpinned beyond 1 ulp;
+ *   flash attention                                : the reference's own check input
+ *       (every element 0.625 -> every output 0.625, flash_attention_fwd.mlir:481-485)
+ *       and closed forms (one-hot scores, uniform scores = mean of V);
  *   loop fusion / input fusion chains             : parity unpinned by reference
  *       tests (the benchmarks feed constants and check nothing); pinned by closed
  *       forms against an f64 evaluation.
@@ -67,6 +70,9 @@ void oracle_silu_f32(const float *x, float *y, size_t n);              /* benchm
 float oracle_silu_scalar_f32(float x);
 void oracle_loop_fusion_f32(const float *a, const float *b, float *out, size_t n);                    /* benchmarks/kLoopFusion/kLoopFusion.mlir.in:6-29 */
 void oracle_input_fusion_f32(const float *a, const float *b, float *out, int64_t rows, int64_t cols); /* benchmarks/kInputFusion/kInputFusion.mlir.in:8-39 */
+void oracle_flash_attention_rows(const uint16_t *Q, const uint16_t *K, const uint16_t *V, uint16_t *out_rows,
+                                 int64_t n_ctx, int64_t d_head, float sm_scale, const int64_t *rows,
+                                 int64_t nrows); /* WG/flash_attention_fwd.mlir:332-421 */
 void oracle_logf_n(const float *in, float *out, size_t n);              /* the host libm logf the fused chains call */
 float oracle_expf_cr(float x);                                          /* correctly rounded exp via f64 */
 void oracle_expf_n(const float *in, float *out, size_t n);              /* the host libm expf the oracle's silu/softmax call */

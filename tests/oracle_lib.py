@@ -183,6 +183,17 @@ def input_fusion_f32(a, b):
     return out
 
 
+def flash_attention_rows(q, k, v, n_ctx, sm_scale, rows):
+    """f16 bit patterns [(ZH*n_ctx), d]; returns the f16 bit patterns of the listed rows."""
+    q, k, v = _c(q, np.uint16), _c(k, np.uint16), _c(v, np.uint16)
+    rows = _c(np.asarray(rows), np.int64)
+    d = q.shape[1]
+    out = np.empty((rows.size, d), np.uint16)
+    lib().oracle_flash_attention_rows(_p(q), _p(k), _p(v), _p(out), C.c_int64(n_ctx), C.c_int64(d),
+                                      C.c_float(sm_scale), _p(rows), C.c_int64(rows.size))
+    return out
+
+
 def logf(x):
     x = _c(x, np.float32)
     out = np.empty_like(x)

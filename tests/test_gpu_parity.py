@@ -276,6 +276,66 @@ def test_input_fusion_16bit(host, orc, stream, dtype):
     assert np.array_equal(got, want)
 
 
+# ============================ flash attention ===============================
+def attention_close(got_bits, ref_bits, orc):
+    """The reference checks its kernel with allclose (atol 1e-4, rtol 1e-3) on a constant
+    input.  On random inputs the kernel (P truncated to f16 before normalisation, keys
+    in blocks) and the CPU loop (P truncated after normalisation, keys in order) differ
+    by f16 roundings of P, each <= 2^-11 relative: |d| <= 2^-10 * max|V| plus one f16
+    output rounding."""
+    got, ref = orc.half_to_float(got_bits), orc.half_to_float(ref_bits)
+    return np.max(np.abs(got - ref)) <= 2.0 ** -10 + 2.0 ** -11 * np.max(np.abs(ref))
+
+
+@pytest.mark.parametrize("zh,n_ctx", [(1, 128), (3, 256), (2, 1024), (2, 100), (1, 64)])
+def test_flash_attention_vs_oracle(host, orc, stream, zh, n_ctx):
+    n = zh * n_ctx
+    q = orc.fill_uniform(n * 64, "f16", 51, -1, 1).reshape(n, 64)
+    k = orc.fill_uniform(n * 64, "f16", 52, -1, 1).reshape(n, 64)
+    v = orc.fill_uniform(n * 64, "f16", 53, -1, 1).reshape(n, 64)
+    got = host.flash_attention(stream, q, k, v, zh, n_ctx, 0.5)
+    rows = np.arange(n) if n <= 512 else np.unique(np.concatenate([np.arange(0, n, 37), [n_ctx - 1, n_ctx, n - 1]]))
+    ref = orc.flash_attention_rows(q, k, v, n_ctx, 0.5, rows)
+    assert attention_close(got[rows], ref, orc)
+
+
+def test_flash_attention_sharp_scores(host, orc, stream):
+    """Large score range (scale 4, |q.k| up to ~20): the running max changes from block
+    to block and the rescaling of the accumulator is exercised."""
+    zh, n_ctx = 2, 512
+    n = zh * n_ctx
+    q = orc.fill_uniform(n * 64, "f16", 54, -2, 2).reshape(n, 64)
+    k = orc.fill_uniform(n * 64, "f16", 55, -2, 2).reshape(n, 64)
+    v = orc.fill_uniform(n * 64, "f16", 56, -1, 1).reshape(n, 64)
+    got = host.flash_attention(stream, q, k, v, zh, n_ctx, 4.0)
+    rows = np.arange(0, n, 5)
+    assert attention_close(got[rows], orc.flash_attention_rows(q, k, v, n_ctx, 4.0, rows), orc)
+
+
+def test_flash_attention_reference_config(host, orc, stream):
+    """Z = 2, H = 2, N_CTX = 4096, D = 64, scale 0.5 (flash_attention_fwd.mlir:449-454):
+    the reference's own constant input exactly, then random inputs on sampled rows."""
+    zh, n_ctx = 4, 4096
+    n = zh * n_ctx
+    const = orc.from_float(np.full((n, 64), 0.625, np.float32), "f16")
+    out = host.flash_attention(stream, const, const, const, zh, n_ctx, 0.5)
+    assert np.all(orc.half_to_float(out) == 0.625)
+    q = orc.fill_uniform(n * 64, "f16", 57, -1, 1).reshape(n, 64)
+    k = orc.fill_uniform(n * 64, "f16", 58, -1, 1).reshape(n, 64)
+    v = orc.fill_uniform(n * 64, "f16", 59, -1, 1).reshape(n, 64)
+    got = host.flash_attention(stream, q, k, v, zh, n_ctx, 0.5)
+    rows = np.array([0, 1, 63, 64, 4095, 4096, 5000, 8191, 8192, 12287, 12288, 16383])
+    ref = orc.flash_attention_rows(q, k, v, n_ctx, 0.5, rows)
+    assert attention_close(got[rows], ref, orc)
+    # permuting the keys (and values with them) of one head leaves its outputs unchanged up to rounding
+    perm = np.random.default_rng(3).permutation(n_ctx)
+    k2, v2 = k.copy(), v.copy()
+    k2[:n_ctx], v2[:n_ctx] = k[:n_ctx][perm], v[:n_ctx][perm]
+    got2 = host.flash_attention(stream, q, k2, v2, zh, n_ctx, 0.5)
+    assert attention_close(got2[:n_ctx], got[:n_ctx], orc)
+    assert np.array_equal(got2[n_ctx:], got[n_ctx:])
+
+
 # =============================== GEMM ======================================
 def gemm_close(got, ref):
     return np.max(np.abs(got - ref)) <= 5e-3 * np.max(np.abs(ref))

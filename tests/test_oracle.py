@@ -215,6 +215,41 @@ def test_fused_chains_closed_forms(orc):
     assert np.all(c == acc)
 
 
+# ---- flash attention -----------------------------------------------------------------
+def test_flash_attention_reference_closed_forms(orc):
+    n_ctx, d = 256, 64
+    f16 = lambda a: orc.from_float(np.asarray(a, np.float32), "f16")
+    # the reference's own check input: every element 0.625 -> uniform softmax -> every output 0.625
+    # (WG/flash_attention_fwd.mlir:481-485, checked there with allclose)
+    x = f16(np.full((2 * n_ctx, d), 0.625))
+    out = orc.flash_attention_rows(x, x, x, n_ctx, 0.5, np.arange(2 * n_ctx))
+    assert np.all(orc.half_to_float(out) == 0.625)
+    # K = 0: uniform probabilities 1/256 (exact in f16), output = f16(mean of V) per head
+    rng = np.random.default_rng(5)
+    q = f16(rng.uniform(-1, 1, (2 * n_ctx, d)))
+    v = f16(rng.uniform(-1, 1, (2 * n_ctx, d)))
+    out = orc.half_to_float(orc.flash_attention_rows(q, f16(np.zeros((2 * n_ctx, d))), v, n_ctx, 0.5, [0, 300]))
+    vf = orc.half_to_float(v).astype(np.float64)
+    assert np.max(np.abs(out[0] - vf[:n_ctx].mean(axis=0))) < 2e-3      # row 0 belongs to head 0
+    assert np.max(np.abs(out[1] - vf[n_ctx:].mean(axis=0))) < 2e-3      # row 300 to head 1: heads do not mix
+    # one dominant key: q = 8 e_0, key 77 = 8 e_0, others 0 -> score 32 at key 77 -> output = V[77]
+    qh = np.zeros((n_ctx, d), np.float32); qh[:, 0] = 8.0
+    kh = np.zeros((n_ctx, d), np.float32); kh[77, 0] = 8.0
+    v1 = f16(rng.uniform(-1, 1, (n_ctx, d)))
+    out = orc.flash_attention_rows(f16(qh), f16(kh), v1, n_ctx, 1.0, [5])
+    assert np.max(np.abs(orc.half_to_float(out)[0] - orc.half_to_float(v1)[77])) < 1e-3
+    # general case against an f64 evaluation
+    k = f16(rng.uniform(-1, 1, (2 * n_ctx, d)))
+    rows = np.array([0, 17, 255, 256, 511])
+    got = orc.half_to_float(orc.flash_attention_rows(q, k, v, n_ctx, 0.5, rows)).astype(np.float64)
+    qf, kf = orc.half_to_float(q).astype(np.float64), orc.half_to_float(k).astype(np.float64)
+    for i, r in enumerate(rows):
+        h = r // n_ctx
+        s = 0.5 * kf[h * n_ctx:(h + 1) * n_ctx] @ qf[r]
+        p = np.exp(s - s.max()); p /= p.sum()
+        assert np.max(np.abs(got[i] - p @ vf[h * n_ctx:(h + 1) * n_ctx])) < 1e-3
+
+
 # ---- softmax ---------------------------------------------------------------------
 @pytest.mark.parametrize("key", ["softmax_f32_10x20", "softmax_f32_10x20_spirv"])
 def test_softmax_golden(orc, key):
