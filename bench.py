@@ -187,7 +187,10 @@ def roofline(w, ms):
 def measure_secondary(stream, w, rounds):
     """Back-to-back launches (one event pair around all of them) and the
     IMEX-profiler protocol with a cache flush before each timed launch."""
-    hot_total = stream.profile(w.kernel, w.dims, w.args, warmups=3, rounds=rounds, mode=1)[0]
+    # MFMA-bound kernels get a long warm-up: coming from lighter work the part needs
+    # ~100 launches before its clock settles under the new load
+    warm = 150 if w.bound == "mfma" else 3
+    hot_total = stream.profile(w.kernel, w.dims, w.args, warmups=warm, rounds=rounds, mode=1)[0]
     hot_ms = hot_total / rounds
     cold = stream.profile(w.kernel, w.dims, w.args, warmups=2, rounds=min(rounds, 20), flush_bytes=FLUSH_BYTES, mode=0)
     cold_ms = float(np.median(cold))
