@@ -21,17 +21,18 @@
 // plain register loops plus ONE exchange between lane l and l+32 per block of
 // keys.
 //
-// Workgroup = 64 queries of one (batch, head): 4 wavefronts = 2 query halves x 2
-// key parities (wavefront w takes queries 32*(w&1).. and every second 64-key
-// tile, parity w>>1), partial (m, l, O) of the two parities merged through LDS at
-// the end.  That keeps 256 workgroups in flight for the reference's shape
+// Workgroup = 64 queries of one (batch, head): 8 wavefronts = 2 query halves x 4
+// key groups (wavefront w takes queries 32*(w&1).. and every fourth 64-key tile,
+// group w>>1), partial (m, l, O) of the four groups merged through LDS at the
+// end.  That keeps 256 workgroups in flight for the reference's shape
 // (2 x 2 x 4096 x 64: one per CU) where a 128-query tile would fill half the
-// chip.  K and V tiles of 128 keys (both parities) go from global memory straight
-// into a three-stage LDS ring (buffer_load ... lds), two iterations ahead.
+// chip, and puts two wavefronts on every SIMD, so one's MFMAs run under the
+// other's exponentials.  K and V blocks of 256 keys go from global memory straight
+// into a two-stage LDS ring (buffer_load ... lds), one block ahead.
 //
 // Arguments: (Q, K, V, Out, sm_scale: f32, ZH: i64, N_CTX: i64)   dims = {ZH, N_CTX}
-//   ZH = batch * heads; N_CTX a multiple of 128; all four tensors [(ZH*N_CTX), 64].
-// Launch: block (256,1,1); grid (N_CTX/64, ZH, 1).  Other shapes take the
+//   ZH = batch * heads; N_CTX a multiple of 256; all four tensors [(ZH*N_CTX), 64].
+// Launch: block (512,1,1); grid (N_CTX/64, ZH, 1).  Other shapes take the
 // one-query-per-lane reference loop of the same kernel (grid-stride, any grid).
 
 #include "device_common.h"
@@ -40,14 +41,16 @@ using namespace imexhip;
 
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
+constexpr int kWaves = kThreads / 64;
+constexpr int kKeyGroups = kWaves / 2;  // wavefronts that split the keys of one query half
 constexpr int D = 64;                 // head dimension
 constexpr int BM = 64;                // queries per workgroup
-constexpr int BN = 64;                // keys per tile; a ring stage holds two tiles (one per parity)
+constexpr int BN = 64;                // keys per tile; a ring stage holds one tile per key group
 constexpr int kTileBytes = BN * D * 2;          // 8 KiB
-constexpr int kStageBytes = 4 * kTileBytes;     // K0, K1, V0, V1 = 32 KiB
-constexpr int kStages = 3;
-constexpr int kDmaPerWave = kStageBytes / 1024 / 4; // 8 copies of 1 KiB per wavefront and stage
+constexpr int kStageBytes = 2 * kKeyGroups * kTileBytes; // K0..K3, V0..V3 = 64 KiB
+constexpr int kStages = 2;
+constexpr int kDmaPerWave = kStageBytes / 1024 / kWaves; // 8 copies of 1 KiB per wavefront and stage
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
@@ -126,23 +129,23 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
   int kVoff[4], vVoff[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
-    // wavefront w copies rows [32w, 32w+32) of the stage's 128 K rows and of its 128 V rows
-    const int row = wave * 32 + c * 8 + (lane >> 3); // 0..127: key within the 128-key stage
+    // wavefront w copies rows [32w, 32w+32) of the stage's 256 K rows and of its 256 V rows
+    const int row = wave * 32 + c * 8 + (lane >> 3); // 0..255: key within the 256-key stage
     const int r = row & 63;                          // row within its tile
     const int kc = (lane & 7) ^ ((r ^ ((r >> 3) & 3)) & 7);
     const int vc = (lane & 7) ^ (((r >> 1) & 1) << 2);
     kVoff[c] = (row * D + kc * 8) * 2;
     vVoff[c] = (row * D + vc * 8) * 2;
   }
-  auto dma_stage = [&](int it, int stageOff) { // keys [128 it, 128 it + 128)
+  auto dma_stage = [&](int it, int stageOff) { // keys [256 it, 256 it + 256)
     LdsChar *dst = ldsBase + stageOff + wave * 4096;
-    const int soff = it * (2 * BN * D * 2);
+    const int soff = it * (kKeyGroups * BN * D * 2);
 #pragma unroll
     for (int c = 0; c < 4; ++c)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(kRsrc, dst + c * 1024, 16, kVoff[c], soff, 0, 0);
 #pragma unroll
     for (int c = 0; c < 4; ++c)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(vRsrc, dst + 2 * kTileBytes + c * 1024, 16, vVoff[c], soff, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vRsrc, dst + kKeyGroups * kTileBytes + c * 1024, 16, vVoff[c], soff, 0, 0);
   };
 
   // -- LDS read addresses (relative to this wavefront's K / V tile of a stage)
@@ -164,7 +167,7 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
 #pragma unroll
     for (int db = 0; db < 2; ++db) {
       const int chunk = ((db ^ ((t >> 3) & 1)) << 2) | (blk << 1) | ((t & 3) >> 1);
-      vRd[db] = 2 * kTileBytes + wk * kTileBytes + row * 128 + chunk * 16 + (t & 1) * 8;
+      vRd[db] = kKeyGroups * kTileBytes + wk * kTileBytes + row * 128 + chunk * 16 + (t & 1) * 8;
     }
   }
 
@@ -178,15 +181,14 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
   float l = 0.0f;              // running sum of p over THIS lane's keys only
   const float c = scale * 1.44269504088896341f;
 
-  const int iters = int(N / (2 * BN));
+  const int iters = int(N / (kKeyGroups * BN));
   dma_stage(0, 0);
-  dma_stage(min(1, iters - 1), kStageBytes);
-  int curOff = 0, dmaOff = 2 * kStageBytes;
+  int curOff = 0;
   for (int it = 0; it < iters; ++it) {
-    wait_vmcnt<kDmaPerWave>(); // stage `it` has landed (this wavefront's copies); the next one may be in flight
-    __builtin_amdgcn_s_barrier(); // ... everyone's; and everyone is done reading stage it-1
+    wait_vmcnt<0>();              // block `it` has landed (this wavefront's copies)
+    __builtin_amdgcn_s_barrier(); // ... everyone's; and everyone is done reading block it-1
     __builtin_amdgcn_sched_barrier(0);
-    dma_stage(min(it + 2, iters - 1), dmaOff); // into the stage read in iteration it-1
+    dma_stage(min(it + 1, iters - 1), curOff ^ kStageBytes); // into the stage block it-1 occupied
     const char *st = lds + curOff;
 
     // S^T = K . Q^T for this wavefront's 64 keys
@@ -242,42 +244,56 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
         o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[kk], o[db], 0, 0, 0);
       }
     }
-    curOff = curOff + kStageBytes == kStages * kStageBytes ? 0 : curOff + kStageBytes;
-    dmaOff = dmaOff + kStageBytes == kStages * kStageBytes ? 0 : dmaOff + kStageBytes;
+    curOff ^= kStageBytes;
   }
   wait_vmcnt<0>();
   l += other_half(l); // both key halves of the lane pair
 
-  // -- merge the two key parities through LDS: wavefronts 2,3 hand (m, l, O^T) to 0,1
+  // -- merge the key groups through LDS: groups 1.. hand (m, l, O^T) to group 0
   __syncthreads(); // the ring is free
-  float *xchg = reinterpret_cast<float *>(lds) + wq * (64 * 34);
-  if (wk == 1) {
+  constexpr int kSlot = 34 * 64; // floats per (query half, key group): 32 accumulator rows, m, l
+  float *xchg = reinterpret_cast<float *>(lds) + wq * (kKeyGroups - 1) * kSlot;
+  if (wk != 0) {
+    float *mine = xchg + (wk - 1) * kSlot;
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        xchg[(db * 16 + r) * 64 + lane] = o[db][r];
-    xchg[32 * 64 + lane] = m;
-    xchg[33 * 64 + lane] = l;
+        mine[(db * 16 + r) * 64 + lane] = o[db][r];
+    mine[32 * 64 + lane] = m;
+    mine[33 * 64 + lane] = l;
   }
   __syncthreads();
   if (wk == 0) {
-    const float m1 = xchg[32 * 64 + lane], l1 = xchg[33 * 64 + lane];
-    const float mAll = fmaxf(m, m1);
-    const float a0 = exp2f(m - mAll), a1 = exp2f(m1 - mAll);
-    const float inv = 1.0f / (l * a0 + l1 * a1);
+    float mAll = m;
+#pragma unroll
+    for (int g = 0; g < kKeyGroups - 1; ++g)
+      mAll = fmaxf(mAll, xchg[g * kSlot + 32 * 64 + lane]);
+    float a[kKeyGroups];
+    a[0] = exp2f(m - mAll);
+    float lAll = l * a[0];
+#pragma unroll
+    for (int g = 0; g < kKeyGroups - 1; ++g) {
+      a[g + 1] = exp2f(xchg[g * kSlot + 32 * 64 + lane] - mAll);
+      lAll += xchg[g * kSlot + 33 * 64 + lane] * a[g + 1];
+    }
+    const float inv = 1.0f / lAll;
     // lane holds, for query q = qi, d = db*32 + (r/4)*8 + half*4 + r%4
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int g4 = 0; g4 < 4; ++g4) {
         f16x4 out4;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int r = g * 4 + e;
-          out4[e] = static_cast<_Float16>((o[db][r] * a0 + xchg[(db * 16 + r) * 64 + lane] * a1) * inv);
+          const int r = g4 * 4 + e;
+          float acc = o[db][r] * a[0];
+#pragma unroll
+          for (int g = 0; g < kKeyGroups - 1; ++g)
+            acc += xchg[g * kSlot + (db * 16 + r) * 64 + lane] * a[g + 1];
+          out4[e] = static_cast<_Float16>(acc * inv);
         }
-        *reinterpret_cast<f16x4 *>(Out + (q0 + qi) * D + db * 32 + g * 8 + half * 4) = out4;
+        *reinterpret_cast<f16x4 *>(Out + (q0 + qi) * D + db * 32 + g4 * 8 + half * 4) = out4;
       }
   }
 }
@@ -290,7 +306,7 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_flash_attention_fwd_
                                                                                    uint16_t *Out, float sm_scale,
                                                                                    int64_t ZH, int64_t N_CTX) {
   __shared__ __attribute__((aligned(16))) char lds[kStages * kStageBytes];
-  const bool tileable = N_CTX > 0 && N_CTX % (2 * BN) == 0 && gridDim.x == N_CTX / BM && gridDim.y == ZH &&
+  const bool tileable = N_CTX > 0 && N_CTX % (kKeyGroups * BN) == 0 && gridDim.x == N_CTX / BM && gridDim.y == ZH &&
                         gridDim.z == 1 &&
                         ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
                           reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(Out)) & 15) == 0;

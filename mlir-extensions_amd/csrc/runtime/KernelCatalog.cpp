@@ -182,13 +182,14 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     grid[2] = static_cast<size_t>(dims[1]);
     break;
   }
-  case Shape::Attention: { // dims = {ZH, N_CTX}; 64 queries per workgroup when N_CTX % 128 == 0
+  case Shape::Attention: { // dims = {ZH, N_CTX}; 64 queries x 8 wavefronts per workgroup when N_CTX % 256 == 0
     const int64_t ZH = dims[0], N = dims[1];
-    if (N > 0 && N % 128 == 0 && ZH > 0 && ZH <= 65535) {
+    block[0] = 512;
+    if (N > 0 && N % 256 == 0 && ZH > 0 && ZH <= 65535) {
       grid[0] = static_cast<size_t>(N / 64);
       grid[1] = static_cast<size_t>(ZH);
     } else {
-      grid[0] = ceilDiv(ZH * N, 256); // one lane per query
+      grid[0] = ceilDiv(ZH * N, 512); // one lane per query
     }
     break;
   }

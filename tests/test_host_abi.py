@@ -81,7 +81,7 @@ def test_launch_shapes(host):
     assert ls("imex_gemm_f16_f16_f32", [256, 256, 48])[0] == (128, 1, 1)
     assert ls("imex_gemm_f16_f16_f32", [255, 256, 64])[0] == (128, 1, 1)
     assert ls("imex_gemm_4kx4kx4k_f16_f16_f32", []) == ((16, 16, 1), (512, 1, 1), 0)
-    assert ls("imex_flash_attention_fwd_f16", [4, 4096]) == ((64, 4, 1), (256, 1, 1), 0)
+    assert ls("imex_flash_attention_fwd_f16", [4, 4096]) == ((64, 4, 1), (512, 1, 1), 0)
     assert ls("imex_flash_attention_fwd_f16", [2, 100])[0] == (1, 1, 1)
     assert ls("imex_input_fusion_f32", [512, 1024])[0] == (4, 1, 1)
     assert ls("imex_gemm_4kx4kx4k_transpose_a", []) == ((16, 16, 1), (512, 1, 1), 0)
