@@ -167,19 +167,27 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
   case Shape::ReduceOuter: // four outputs per lane
     grid[0] = ceilDiv(dims[1], 1024);
     break;
-  case Shape::Transpose2D32: // 64 x 64 tiles
-  case Shape::Transpose2D16: { // 128 x 128 tiles
-    const int64_t tile = e->shape == Shape::Transpose2D32 ? 64 : 128;
-    grid[0] = ceilDiv(dims[1], tile);
-    grid[1] = ceilDiv(dims[0], tile);
-    break;
-  }
+  case Shape::Transpose2D32:
+  case Shape::Transpose2D16:
   case Shape::Transpose3D32:
   case Shape::Transpose3D16: {
-    const int64_t tile = e->shape == Shape::Transpose3D32 ? 64 : 128;
-    grid[0] = ceilDiv(dims[2], tile);
-    grid[1] = ceilDiv(dims[0], tile);
-    grid[2] = static_cast<size_t>(dims[1]);
+    // One workgroup per R x C tile.  Problems of 2^24 elements and more use the
+    // large tiles (512-byte row segments): 128 x 128 for 32-bit, 256 x 256 for
+    // 16-bit elements; smaller ones 64 x 64 / 128 x 128.  The kernels apply the same
+    // rule, and stride over the tiles if the grid is any different.
+    const bool is32 = e->shape == Shape::Transpose2D32 || e->shape == Shape::Transpose3D32;
+    const bool is3d = e->shape == Shape::Transpose3D32 || e->shape == Shape::Transpose3D16;
+    const int64_t rows = dims[0], cols = is3d ? dims[2] : dims[1], planes = is3d ? dims[1] : 1;
+    const bool big = rows * cols * planes >= (int64_t(1) << 24);
+    const int64_t tileR = is32 ? (big ? 128 : 64) : (big ? 256 : 128);
+    const int64_t tileC = is32 ? (big ? 128 : 64) : (big ? 256 : 128);
+    grid[0] = ceilDiv(cols, tileC);
+    grid[1] = ceilDiv(rows, tileR);
+    grid[2] = static_cast<size_t>(planes);
+    if (grid[1] > 65535) // the kernels stride over the tiles a smaller grid leaves out
+      grid[1] = 65535;
+    if (grid[2] > 65535)
+      grid[2] = 65535;
     break;
   }
   case Shape::Attention: { // dims = {ZH, N_CTX}; 64 queries x 8 wavefronts per workgroup when N_CTX % 256 == 0

@@ -209,7 +209,36 @@ def test_transpose_config_sizes(host, orc, stream):
     assert np.array_equal(host.transpose2d(stream, y), orc.transpose2d(y))
 
 
-@pytest.mark.parametrize("shape", [(16, 96, 96), (96, 7, 96), (5, 3, 9), (64, 2, 72)])
+@pytest.mark.parametrize("rows,cols", [(4104, 4120), (8200, 2056), (300, 65544)])
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_transpose_large_tiles_ragged(host, orc, stream, rows, cols, dtype):
+    """From 2^24 elements the kernels use 128 x 128 (32-bit) / 256 x 128 (16-bit)
+    tiles; these shapes end in partial tiles on both sides."""
+    x = orc.fill_bits(rows * cols, dtype, 20244 + cols).reshape(rows, cols)
+    got = host.transpose2d(stream, x)
+    assert np.array_equal(got, x.T)
+
+
+def test_transpose_any_grid(host, orc, stream):
+    """Workgroups stride over the tiles: a grid smaller or larger than one workgroup
+    per tile gives the same result."""
+    import ctypes as C
+    for name, np_t, rows, cols in [("imex_transpose2d_b32", np.uint32, 4096, 4104), ("imex_transpose2d_b16", np.uint16, 520, 264)]:
+        x = np.arange(rows * cols, dtype=np.uint64).astype(np_t).reshape(rows, cols)
+        for grid in [(3, 1, 1), (7, 5, 2)]:
+            d_in, d_out = stream.to_device(x), stream.alloc(x.nbytes)
+            fn = stream.kernel(name)
+            descs, keep = host._pack_params([d_in, d_out, rows, cols])
+            stream.rt.gpuLaunchKernel(stream.handle, fn, grid[0], grid[1], grid[2], 256, 1, 1, 0,
+                                      C.cast(descs, C.c_void_p), None)
+            stream.wait()
+            got = stream.from_device(d_out, (cols, rows), np_t)
+            stream.free(d_in)
+            stream.free(d_out)
+            assert np.array_equal(got, x.T), (name, grid)
+
+
+@pytest.mark.parametrize("shape", [(16, 96, 96), (96, 7, 96), (5, 3, 9), (64, 2, 72), (520, 64, 512)])
 def test_transpose3d(host, orc, stream, shape):
     n = int(np.prod(shape))
     x32 = orc.fill_bits(n, "f32", 5).reshape(shape)

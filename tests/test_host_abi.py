@@ -68,8 +68,10 @@ def test_launch_shapes(host):
     assert ls("imex_rowsum_f32", [8192, 8192])[0] == (8192, 1, 1)
     assert ls("imex_rowsum_f32", [8, 256])[0] == (2, 1, 1)
     assert ls("imex_reduce_outer_f32", [32, 16 * 512 * 512])[0] == (4096, 1, 1)
-    assert ls("imex_transpose2d_b16", [8192, 8192])[0] == (64, 64, 1)
-    assert ls("imex_transpose2d_b32", [4096, 4096])[0] == (64, 64, 1)
+    assert ls("imex_transpose2d_b16", [8192, 8192])[0] == (32, 32, 1)   # 256 x 256 tiles from 2^24 elements
+    assert ls("imex_transpose2d_b16", [2048, 2048])[0] == (16, 16, 1)   # 128 x 128 below
+    assert ls("imex_transpose2d_b32", [4096, 4096])[0] == (32, 32, 1)   # 128 x 128 tiles from 2^24 elements
+    assert ls("imex_transpose2d_b32", [2048, 4096])[0] == (64, 32, 1)   # 64 x 64 below
     assert ls("imex_transpose2d_b32", [10, 20])[0] == (1, 1, 1)
     assert ls("imex_transpose3d_b32", [16, 96, 96])[0] == (2, 1, 96)
     assert ls("imex_gemm_f16_f16_f32", [4096, 4096, 4096]) == ((256, 1, 1), (512, 1, 1), 0)
