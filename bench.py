@@ -4,12 +4,14 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME,...] [--no-cpu]
 
 A "step" is one launch of the headline kernel -- the f16 4096^3 GEMM, the
-workload the reference's published numbers and BASELINE's MFMA target are quoted
-on -- over synthetic seeded inputs already resident in HBM.  K steps are timed
-between two stream synchronisations; the same region is also timed with HIP
-events on the launch stream (the events gpuLaunchKernel returns).  Every other
-BASELINE config is measured too and reported under "per_config", each with its
-own roofline fraction and single-core CPU baseline.
+workload the MFMA target of BASELINE.json is quoted on -- over synthetic seeded
+inputs already resident in HBM.  K steps are timed between two stream
+synchronisations; the same region is also timed with HIP events recorded on the
+launch stream through the C ABI.  Every other configuration of BASELINE.json is
+measured too and reported under "per_config" under three protocols (the same
+buffers back to back, a ring of buffer sets larger than every cache, and the
+reference profiler's cache flush before each launch), each with its roofline
+fraction and a single-core CPU baseline.
 
 Prints ONE JSON line.
 """
@@ -38,7 +40,7 @@ def log(msg):
 
 
 class Workload:
-    """One BASELINE config: device buffers, the kernel launch, its algorithmic
+    """One BASELINE.json configuration: device buffers, the kernel launch, its algorithmic
     work and the matching CPU-baseline call."""
 
     def __init__(self, name, kernel, dims, bound, work, unit, dtype, describe):
@@ -320,7 +322,7 @@ def main():
         "metric": METRIC, "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic (seeded std::mt19937 stream, inputs resident in HBM)",
-        "config": {"workload": "BASELINE configs[3]: " + head.describe, "kernel": head.kernel,
+        "config": {"workload": "BASELINE.json configs[3]: " + head.describe, "kernel": head.kernel,
                    "launch": "grid (256,1,1) x block (512,1,1)", "device": info["name"],
                    "cus": info["cus"], "clock_mhz": info["clock_khz"] / 1e3,
                    "gpuMemCopy_h2d_GBps": round(h2d_gbs, 1)},
