@@ -191,17 +191,16 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
     dma_stage(min(it + 1, iters - 1), curOff ^ kStageBytes); // into the stage block it-1 occupied
     const char *st = lds + curOff;
 
-    // S^T = K . Q^T for this wavefront's 64 keys
+    // S^T = K . Q^T for this wavefront's 64 keys (the first product of each chain takes a
+    // literal zero accumulator, so no registers are cleared)
     f32x16 s[2];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        s[kb][r] = 0.0f;
+      const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int ds = 0; ds < 4; ++ds) {
         const f16x8 kf = *reinterpret_cast<const f16x8 *>(st + kRd[ds] + kb * 32 * 128);
-        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ds], s[kb], 0, 0, 0);
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ds], ds == 0 ? zero : s[kb], 0, 0, 0);
       }
     }
     // online softmax over the keys; this lane owns 32 of the query's 64 scores
@@ -221,17 +220,19 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
     for (int kk = 0; kk < 4; ++kk) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = __builtin_amdgcn_exp2f(s[kk >> 1][(kk & 1) * 8 + e] * c - mNew);
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kk >> 1][(kk & 1) * 8 + e], c, -mNew)); // one fused op per score
         pf[kk][e] = static_cast<_Float16>(p); // the reference truncates P to f16 before P.V (:262-265)
         sum += p;                             // ... and sums the untruncated f32 values (:243-247)
       }
     }
     l = l * alpha + sum;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) { // the running max moved for some query of this wavefront
 #pragma unroll
-    for (int db = 0; db < 2; ++db)
+      for (int db = 0; db < 2; ++db)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        o[db][r] *= alpha;
+        for (int r = 0; r < 16; ++r)
+          o[db][r] *= alpha;
+    }
     // O^T += V^T . P^T
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
