@@ -194,14 +194,20 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
     // S^T = K . Q^T for this wavefront's 64 keys (the first product of each chain takes a
     // literal zero accumulator, so no registers are cleared)
     f32x16 s[2];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+    {
       const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+      f16x8 kf[2][4];
 #pragma unroll
-      for (int ds = 0; ds < 4; ++ds) {
-        const f16x8 kf = *reinterpret_cast<const f16x8 *>(st + kRd[ds] + kb * 32 * 128);
-        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ds], ds == 0 ? zero : s[kb], 0, 0, 0);
-      }
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int ds = 0; ds < 4; ++ds)
+          kf[kb][ds] = *reinterpret_cast<const f16x8 *>(st + kRd[ds] + kb * 32 * 128);
+      // the two accumulator chains alternate, so no MFMA waits for the one just issued
+#pragma unroll
+      for (int ds = 0; ds < 4; ++ds)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+          s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[kb][ds], qf[ds], ds == 0 ? zero : s[kb], 0, 0, 0);
     }
     // online softmax over the keys; this lane owns 32 of the query's 64 scores
     float mx = s[0][0];
