@@ -15,7 +15,12 @@
 //
 //   imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--launch-only N] <workload>...
 //   imex-hip-bench --list
+//   imex-hip-bench [-l] --report report.txt <workload>...|all
 //
+//   --report FILE  bench_imex's outer loop (bench_imex.in:72-91): one child process per workload,
+//                  their output echoed, every "execution time" line collected in FILE under an
+//                  "Imex Perf (HIP) @ <date>" header.  The parent never touches the GPU.
+//   -c             bench_imex's CPU mode is not offered: the CPU lowering stays IMEX's own pipeline
 //   -l             accepted for bench_imex compatibility (the HIP runtime is the only backend here)
 //   --zeros        all-zero inputs instead of random ones: MFMA power, and with it the clock the
 //                  part sustains, depends on operand values; this shows the kernel at full clock
@@ -31,6 +36,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <ctime>
 #include <string>
 #include <vector>
 
@@ -201,9 +207,46 @@ int runWorkload(const Workload &w, const Options &opt) {
 
 } // namespace
 
+// One child process per workload, as bench_imex runs one mlir-runner per .mlir file.
+int runReport(const char *self, const std::string &reportPath, const std::string &options,
+              const std::vector<std::string> &names) {
+  FILE *report = fopen(reportPath.c_str(), "w");
+  if (!report) {
+    fprintf(stderr, "cannot write %s\n", reportPath.c_str());
+    return 1;
+  }
+  const time_t now = time(nullptr);
+  char date[64];
+  strftime(date, sizeof date, "%a %b %e %H:%M:%S %Z %Y", localtime(&now));
+  fprintf(report, "\n================ Imex Perf (HIP) @ %s ================\n\n", date);
+  int rc = 0;
+  for (const std::string &n : names) {
+    fprintf(stderr, "%s: ", n.c_str());
+    const std::string cmd = std::string("\"") + self + "\"" + options + " " + n;
+    FILE *child = popen(cmd.c_str(), "r");
+    if (!child) {
+      fprintf(stderr, "cannot start %s\n", cmd.c_str());
+      rc = 1;
+      continue;
+    }
+    char line[2048];
+    while (fgets(line, sizeof line, child)) {
+      fputs(line, stdout);
+      if (strstr(line, "execution time"))
+        fputs(line, report); // the driver's lines already start with "<workload>: "
+    }
+    const int status = pclose(child);
+    if (status != 0)
+      rc = 1; // like bench_imex, keep going; the exit code reports that something failed
+  }
+  fclose(report);
+  return rc;
+}
+
 int main(int argc, char **argv) {
   Options opt;
   std::vector<std::string> names;
+  std::string reportPath, childOptions;
   const std::vector<Workload> all = workloads();
   for (int i = 1; i < argc; ++i) {
     const std::string a = argv[i];
@@ -211,16 +254,25 @@ int main(int argc, char **argv) {
       for (const Workload &w : all)
         printf("%s  (%s)\n", w.name, w.kernel);
       return 0;
-    } else if (a == "-l") {
-      // backend selector of bench_imex; HIP is the only one here
+    } else if (a == "-l" || a == "-s") {
+      // backend selectors of bench_imex (Level Zero / SYCL); HIP is the only runtime here
+    } else if (a == "-c") {
+      fprintf(stderr, "-c (CPU lowering) is not part of this library: it stays IMEX's linalg-to-cpu pipeline\n");
+      return 1;
+    } else if (a == "--report" && i + 1 < argc) {
+      reportPath = argv[++i];
     } else if (a == "--flush") {
       opt.flush = true;
+      childOptions += " --flush";
     } else if (a == "--zeros") {
       opt.zeros = true;
+      childOptions += " --zeros";
     } else if (a == "--runs" && i + 1 < argc) {
       opt.runs = atoi(argv[++i]);
+      childOptions += " --runs " + std::to_string(opt.runs);
     } else if (a == "--warmups" && i + 1 < argc) {
       opt.warmups = atoi(argv[++i]);
+      childOptions += " --warmups " + std::to_string(opt.warmups);
     } else if (a == "--launch-only" && i + 1 < argc) {
       opt.launchOnly = atoi(argv[++i]);
     } else if (a == "all") {
@@ -231,10 +283,21 @@ int main(int argc, char **argv) {
     }
   }
   if (names.empty() || opt.runs < 1) {
-    fprintf(stderr, "usage: imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--launch-only N] <workload>|all ...\n"
+    fprintf(stderr, "usage: imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--launch-only N] [--report FILE] <workload>|all ...\n"
                     "       imex-hip-bench --list\n");
     return 2;
   }
+  for (const std::string &n : names) {
+    bool known = false;
+    for (const Workload &w : all)
+      known = known || n == w.name;
+    if (!known) {
+      fprintf(stderr, "unknown workload %s (try --list)\n", n.c_str());
+      return 2;
+    }
+  }
+  if (!reportPath.empty())
+    return runReport(argv[0], reportPath, childOptions, names);
   printf("\n================ Imex Perf (HIP runtime) ================\n\n");
   for (const std::string &n : names) {
     const Workload *found = nullptr;

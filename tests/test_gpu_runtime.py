@@ -154,3 +154,21 @@ def test_mgpu_entry_points(host, orc):
     rt.mgpuMemFree(s, d_in)
     rt.mgpuMemFree(s, d_out)
     rt.mgpuStreamDestroy(s)
+
+
+def test_driver_report_mode(tmp_path):
+    """The C++ driver in bench_imex's role: one child process per workload, their
+    "execution time" lines collected in a report file (benchmarks/bench_imex.in:72-91)."""
+    exe = os.path.join(REPO, "mlir-extensions_amd", "lib", "imex-hip-bench")
+    report = tmp_path / "report.txt"
+    r = subprocess.run([exe, "-l", "--runs", "5", "--warmups", "2", "--report", str(report),
+                        "relu_f32_4096x4096", "softmax_f16_16384x1024"],
+                       stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    lines = report.read_text().splitlines()
+    assert any(l.startswith("================ Imex Perf (HIP) @ ") for l in lines)
+    timed = [l for l in lines if "execution time" in l]
+    assert len(timed) == 2
+    assert timed[0].startswith("relu_f32_4096x4096: the kernel execution time is (ms, on HIP runtime):avg: ")
+    assert timed[1].startswith("softmax_f16_16384x1024: the kernel execution time is (ms, on HIP runtime):avg: ")
+    assert all(l.endswith("(over 5 runs)") for l in timed)

@@ -243,3 +243,18 @@ def test_print_helpers(host, orc, capfd):
     assert "sizes = [3, 3] strides = [3, 1] data =" in out
     assert "[11,   13,   10.5]" in out
     assert "Max absolute error 0" in out
+
+
+def test_driver_command_line():
+    """Parts of the C++ driver that need no GPU: the workload list, bench_imex's -c
+    (not offered) and an unknown workload name."""
+    import subprocess
+    exe = os.path.join(REPO, "mlir-extensions_amd", "lib", "imex-hip-bench")
+    r = subprocess.run([exe, "--list"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+    assert r.returncode == 0
+    names = [l.split()[0] for l in r.stdout.splitlines() if l.strip()]
+    assert "gemm_f16_4096" in names and "flash_attention_f16_2x2x4096x64" in names and len(names) >= 11
+    r = subprocess.run([exe, "-c", "all"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+    assert r.returncode == 1 and "CPU lowering" in r.stderr
+    r = subprocess.run([exe, "no_such_workload"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+    assert r.returncode == 2 and "unknown workload" in r.stderr
