@@ -84,6 +84,9 @@ void *gpuKernelGet(void *queue, void *module, const char *name);
  * bits of sharedMemBytes are used (the call site passes i32).  Returns an
  * event that stands for "after this launch" on the stream, owned by the
  * stream; it can be listed in a later launch's depEvents (on any stream).
+ * The handle is valid until the stream is destroyed; once 4096 further
+ * launches have gone to the stream it stands for a later position of that
+ * stream (a wait on it then waits longer than needed, never shorter).
  * Environment (LevelZeroRuntimeWrappers.cpp:521-597): IMEX_ENABLE_PROFILING,
  * IMEX_PROFILING_RUNS (default 1000), IMEX_PROFILING_WARMUPS (default 3),
  * IMEX_ENABLE_CACHE_FLUSHING, plus IMEX_CACHE_FLUSH_BYTES (default 512 MiB). */

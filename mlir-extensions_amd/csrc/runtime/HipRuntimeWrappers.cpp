@@ -15,9 +15,10 @@
 //    by blob address for the life of the process; kernels are cached per
 //    (module, name), so the load+get pair that precedes every launch costs two
 //    map lookups;
-//  * events returned by gpuLaunchKernel are stream positions, owned by the
-//    stream and released when it is destroyed (the reference never frees
-//    them); the HIP event behind one is recorded only when it is first used;
+//  * events returned by gpuLaunchKernel are stream positions held in a ring of
+//    slots owned by the stream (the reference never frees its events and draws
+//    them from a 256-slot pool that overflows); the HIP event behind one is
+//    recorded only when it is first used;
 //  * profiling uses hipEvent pairs on the launch stream.
 //
 //===----------------------------------------------------------------------===//
@@ -73,16 +74,24 @@ struct GpuHipQueue;
 // dependency on it is satisfied no earlier than the reference semantics demand.
 struct LaunchEvent {
   GpuHipQueue *queue;
-  uint64_t sequence;
-  hipEvent_t event; // null until someone waits on or times this position
+  uint64_t sequence;    // the launch this slot currently stands for
+  hipEvent_t event;     // null until someone waits on or times a position of this slot
+  uint64_t recordedFor; // sequence `event` was last recorded for (0: never)
 };
+
+// Launch events live in a ring: a handle stays valid for the life of its stream,
+// and after kEventSlots further launches it stands for a LATER position of the
+// same in-order stream -- waiting on a stale handle over-synchronises, it never
+// under-synchronises -- so a process that launches for days does not grow.
+constexpr size_t kEventSlots = 4096;
 
 struct GpuHipQueue {
   int device = 0;
   hipStream_t stream = nullptr;
   bool ownsStream = true;
   uint64_t launches = 0;
-  std::vector<LaunchEvent *> events; // handed out by gpuLaunchKernel / imexHipRecordTimestamp
+  std::vector<LaunchEvent> ring;          // handed out by gpuLaunchKernel, slot = launch number mod ring size
+  std::vector<LaunchEvent *> timestamps;  // handed out by imexHipRecordTimestamp; kept until the stream goes
   void *flushBuffer = nullptr;    // scratch for the profiler's cache flush
   size_t flushBytes = 0;
 
@@ -100,7 +109,10 @@ struct GpuHipQueue {
   ~GpuHipQueue() noexcept(false) {
     CHECK_HIP(hipSetDevice(device));
     CHECK_HIP(hipStreamSynchronize(stream));
-    for (LaunchEvent *e : events) {
+    for (LaunchEvent &e : ring)
+      if (e.event)
+        CHECK_HIP(hipEventDestroy(e.event));
+    for (LaunchEvent *e : timestamps) {
       if (e->event)
         CHECK_HIP(hipEventDestroy(e->event));
       delete e;
@@ -382,10 +394,12 @@ long envLong(const char *name, long fallback) {
 }
 
 hipEvent_t materialise(LaunchEvent *le) {
-  if (!le->event) {
+  if (!le->event || le->recordedFor != le->sequence) {
     CHECK_HIP(hipSetDevice(le->queue->device));
-    CHECK_HIP(hipEventCreate(&le->event));
+    if (!le->event)
+      CHECK_HIP(hipEventCreate(&le->event));
     CHECK_HIP(hipEventRecord(le->event, le->queue->stream));
+    le->recordedFor = le->sequence;
   }
   return le->event;
 }
@@ -431,8 +445,10 @@ LaunchEvent *launchKernel(GpuHipQueue *queue, void *kernel, size_t gx, size_t gy
   }
 
   enqueue(queue, la);
-  LaunchEvent *done = new LaunchEvent{queue, ++queue->launches, nullptr};
-  queue->events.push_back(done);
+  if (queue->ring.empty())
+    queue->ring.assign(kEventSlots, LaunchEvent{queue, 0, nullptr, 0});
+  LaunchEvent *done = &queue->ring[queue->launches % kEventSlots];
+  done->sequence = ++queue->launches; // a HIP event left from the slot's previous life is re-recorded on first use
   return done;
 }
 
@@ -603,8 +619,8 @@ extern "C" void *imexHipRecordTimestamp(void *queue) {
     if (!queue)
       throw std::runtime_error("imexHipRecordTimestamp: null stream");
     GpuHipQueue *q = asQueue(queue);
-    LaunchEvent *le = new LaunchEvent{q, q->launches, nullptr};
-    q->events.push_back(le);
+    LaunchEvent *le = new LaunchEvent{q, q->launches + 1, nullptr, 0};
+    q->timestamps.push_back(le);
     materialise(le);
     return le;
   });

@@ -96,6 +96,27 @@ def test_event_dependencies_across_streams(host, orc):
             s1.free(p)
 
 
+def test_launch_events_are_recycled_safely(host, orc):
+    """Launch events come from a 4096-slot ring per stream: a handle older than that
+    still orders a dependent launch after the work it stood for."""
+    n = 4096
+    x = orc.fill_uniform(n, "f32", 9, -1, 1)
+    with host.Stream() as s1, host.Stream() as s2:
+        d_in, d_mid, d_out = s1.to_device(x), s1.alloc(n * 4), s1.alloc(n * 4)
+        step = s1.prepare("imex_relu_f32", [n], [d_in, d_mid, n])
+        first = s1.launch("imex_relu_f32", [n], [d_in, d_mid, n])
+        for _ in range(5000):
+            step()
+        last = s1.launch("imex_silu_f32", [n], [d_in, d_mid, n])
+        assert first and last
+        s2.launch("imex_relu_f32", [n], [d_mid, d_out, n], deps=[first, last])
+        s2.wait()
+        got = s2.from_device(d_out, (n,), np.float32)
+        assert np.array_equal(got, orc.relu_f32(orc.silu_f32(x)))
+        for p in (d_in, d_mid, d_out):
+            s1.free(p)
+
+
 def test_profile_helper_modes(host, orc, stream):
     n = 1 << 22
     d_in, d_out = stream.to_device(orc.fill_uniform(n, "f32", 4, -1, 1)), stream.alloc(n * 4)
