@@ -208,7 +208,7 @@ void copyMemory(GpuHipQueue *queue, void *dst, void *src, size_t bytes) {
 
 // ---- modules and kernels ---------------------------------------------------
 
-std::map<const void *, hipModule_t> moduleCache;
+std::map<std::pair<int, const void *>, hipModule_t> moduleCache; // (device, blob address)
 std::map<std::pair<hipModule_t, std::string>, hipFunction_t> kernelCache;
 std::mutex moduleMutex;
 
@@ -232,23 +232,33 @@ void validateBlob(const void *data, size_t size) {
   const bool compressedBundle = b[0] == 'C' && b[1] == 'C' && b[2] == 'O' && b[3] == 'B';
   if (!elf && !bundle && !compressedBundle)
     throw std::runtime_error("gpuModuleLoad: blob is not a code object (unknown magic)");
+  if (elf) {
+    // e_machine (bytes 18-19, little endian) must be EM_AMDGPU = 224
+    if (size < 20)
+      throw std::runtime_error("gpuModuleLoad: truncated ELF header");
+    const unsigned machine = b[18] | (b[19] << 8);
+    if (machine != 224)
+      throw std::runtime_error("gpuModuleLoad: ELF blob is for machine " + std::to_string(machine) +
+                               ", not an AMDGPU code object");
+  }
 }
 
 hipModule_t loadModule(GpuHipQueue *queue, const void *data, size_t size) {
+  validateBlob(data, size); // a few header bytes; before any HIP call and before the stream is looked at
+  if (!queue)
+    throw std::runtime_error("gpuModuleLoad: null stream");
+  const std::pair<int, const void *> key(queue->device, data);
   {
     std::lock_guard<std::mutex> lock(moduleMutex);
-    auto it = moduleCache.find(data);
+    auto it = moduleCache.find(key);
     if (it != moduleCache.end())
       return it->second;
   }
-  validateBlob(data, size);
-  if (!queue)
-    throw std::runtime_error("gpuModuleLoad: null stream");
   CHECK_HIP(hipSetDevice(queue->device));
   hipModule_t module = nullptr;
   CHECK_HIP(hipModuleLoadData(&module, data));
   std::lock_guard<std::mutex> lock(moduleMutex);
-  auto inserted = moduleCache.emplace(data, module);
+  auto inserted = moduleCache.emplace(key, module);
   if (!inserted.second) { // another thread won the race
     (void)hipModuleUnload(module);
     return inserted.first->second;

@@ -136,6 +136,9 @@ def test_spirv_blob_is_rejected_before_any_gpu_call():
 def test_garbage_and_null_blobs_abort():
     r = _run_snippet("blob = C.create_string_buffer(b'garbage!' * 8)\nrt.gpuModuleLoad(None, blob, 64)\n")
     assert r.returncode == -6 and "not a code object" in r.stdout
+    # an ELF for another machine (x86-64 = 62) is refused by its header, before any HIP call
+    r = _run_snippet("blob = C.create_string_buffer(b'\\x7fELF' + bytes(14) + bytes([62, 0]) + bytes(44))\nrt.gpuModuleLoad(None, blob, 64)\n")
+    assert r.returncode == -6 and "not an AMDGPU code object" in r.stdout
     r = _run_snippet("rt.gpuModuleLoad(None, None, 0)\n")
     assert r.returncode == -6 and "null module data" in r.stdout
     r = _run_snippet("rt.gpuKernelGet(None, None, b'k')\n")
