@@ -272,6 +272,15 @@ def test_loop_fusion_logf_sweep(host, orc, stream):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+def test_fused_chains_empty_and_single(host, orc, stream):
+    empty = np.zeros((0,), np.float32)
+    assert host.loop_fusion(stream, empty, empty).shape == (0,)
+    one = host.loop_fusion(stream, np.float32([2.5]), np.float32([-1.5]))
+    assert np.array_equal(one, orc.loop_fusion_f32(np.float32([2.5]), np.float32([-1.5])))
+    col = host.input_fusion(stream, np.float32([[1.0], [-2.0], [3.0]]), np.float32([[0.5], [2.0], [8.0]]))
+    assert np.array_equal(col, orc.input_fusion_f32(np.float32([[1.0], [-2.0], [3.0]]), np.float32([[0.5], [2.0], [8.0]])))
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_loop_fusion_16bit(host, orc, stream, dtype):
     n = 512 * 1024 + 77
