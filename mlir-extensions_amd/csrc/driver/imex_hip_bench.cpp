@@ -103,6 +103,11 @@ std::vector<Workload> workloads() {
        {{Elem::F16, {4 * K4, 64}, true, -1, 1}, {Elem::F16, {4 * K4, 64}, true, -1, 1},
         {Elem::F16, {4 * K4, 64}, true, -1, 1}, {Elem::F16, {4 * K4, 64}, false, 0, 0}},
        {4, K4}, 2, 4.0 * 4 * K4 * K4 * 64, true},
+      // the reference's second attention shape (flash_attention_fwd_ov_with_arrray_len_4k.mlir:23): 16 heads
+      {"flash_attention_f16_16x4096x64", "imex_flash_attention_fwd_f16", {16, K4},
+       {{Elem::F16, {16 * K4, 64}, true, -1, 1}, {Elem::F16, {16 * K4, 64}, true, -1, 1},
+        {Elem::F16, {16 * K4, 64}, true, -1, 1}, {Elem::F16, {16 * K4, 64}, false, 0, 0}},
+       {16, K4}, 2, 4.0 * 16 * K4 * K4 * 64, true},
   };
 }
 

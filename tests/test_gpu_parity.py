@@ -337,6 +337,20 @@ def test_flash_attention_vs_oracle(host, orc, stream, zh, n_ctx):
     assert attention_close(got[rows], ref, orc)
 
 
+def test_flash_attention_sixteen_heads(host, orc, stream):
+    """16 x 1024 x 64 with the scale 0.350097656 of the reference's second attention
+    test (WG/flash_attention_fwd_ov_with_arrray_len_1k.mlir:22,40; inputs there are
+    uniform(-1,1), checked against a natural-exp softmax)."""
+    zh, n_ctx, scale = 16, 1024, 0.350097656
+    n = zh * n_ctx
+    q = orc.fill_uniform(n * 64, "f16", 61, -1, 1).reshape(n, 64)
+    k = orc.fill_uniform(n * 64, "f16", 62, -1, 1).reshape(n, 64)
+    v = orc.fill_uniform(n * 64, "f16", 63, -1, 1).reshape(n, 64)
+    got = host.flash_attention(stream, q, k, v, zh, n_ctx, scale)
+    rows = np.unique(np.concatenate([np.arange(0, n, 211), [1023, 1024, n - 1]]))
+    assert attention_close(got[rows], orc.flash_attention_rows(q, k, v, n_ctx, scale, rows), orc)
+
+
 def test_flash_attention_sharp_scores(host, orc, stream):
     """Large score range (scale 4, |q.k| up to ~20): the running max changes from block
     to block and the rescaling of the accumulator is exercised."""
