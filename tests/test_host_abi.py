@@ -261,3 +261,46 @@ def test_driver_command_line():
     assert r.returncode == 1 and "CPU lowering" in r.stderr
     r = subprocess.run([exe, "no_such_workload"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
     assert r.returncode == 2 and "unknown workload" in r.stderr
+
+
+def test_launch_shapes_cover_the_problem(host):
+    """For the kernels that do not stride over their work (element-wise, reductions,
+    fused chains, tiled GEMM) the catalogue's grid must cover every element; checked
+    over random problem sizes against each kernel's work per workgroup."""
+    from hypothesis import given, settings, strategies as st
+    ls = host.launch_shape
+
+    @settings(max_examples=300, deadline=None)
+    @given(n=st.integers(1, 1 << 34))
+    def eltwise(n):
+        for name, per in (("imex_relu_f32", 4096), ("imex_silu_f32", 4096), ("imex_relu_bf16", 8192),
+                          ("imex_loop_fusion_f32", 4096), ("imex_loop_fusion_f16", 8192)):
+            (gx, gy, gz), block, _ = ls(name, [n])
+            assert block == (256, 1, 1) and gy == gz == 1
+            assert (gx - 1) * per < n <= gx * per
+
+    @settings(max_examples=300, deadline=None)
+    @given(rows=st.integers(1, 1 << 20), cols=st.integers(1, 1 << 14))
+    def rowwise(rows, cols):
+        (gx, _, _), _, _ = ls("imex_rowsum_f32", [rows, cols])
+        assert gx == rows if cols > 2048 else gx * 4 >= rows
+        (gx, _, _), _, _ = ls("imex_reduce_outer_f32", [rows, cols])
+        assert gx * 1024 >= cols
+        (gx, _, _), _, _ = ls("imex_input_fusion_f32", [rows, cols])
+        assert gx * 256 >= cols
+        (gx, _, _), _, _ = ls("imex_softmax_f16", [rows, cols])
+        assert gx >= 1 and (gx * 4 >= rows if cols <= 1024 else gx >= min(rows, 1048560))
+
+    @settings(max_examples=300, deadline=None)
+    @given(m=st.integers(1, 64), n=st.integers(1, 64), k=st.integers(1, 512), ragged=st.booleans())
+    def gemm(m, n, k, ragged):
+        M, N, K = (m * 256, n * 256, k * 32) if not ragged else (m * 37 + 1, n * 41 + 3, k * 7 + 5)
+        for name in ("imex_gemm_f16_f16_f32", "imex_gemm_f16_f16_f32_ta", "imex_gemm_bf16_bias_silu_bf16"):
+            (gx, gy, gz), block, _ = ls(name, [M, N, K])
+            assert block == (512, 1, 1) and gy == gz == 1
+            tileable = M % 256 == 0 and N % 256 == 0 and K % 32 == 0
+            assert gx == (M // 256) * (N // 256) if tileable else gx * 512 >= M * N
+
+    eltwise()
+    rowwise()
+    gemm()
