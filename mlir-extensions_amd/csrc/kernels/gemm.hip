@@ -1,5 +1,5 @@
 // Tiled MFMA GEMM for gfx950: C[M,N] = A[M,K] . B[K,N], A and B f16 or bf16
-// (row-major), f32 accumulate.
+// (row-major), f32 accumulate; also with A stored [K,M] or B stored [N,K].
 //
 // Reference kernels (workgroup-level XeGPU, the role XeTile's
 // load_tile / prefetch_tile / tile_mma played):
@@ -7,7 +7,9 @@
 //     256x256 workgroup tile, K-step 32, three-deep prefetch, C += A.B;
 //   test/Integration/Dialect/XeGPU/WG/gemm_4kx4kx4k_f16_f16_f32_bias.mlir:77-116
 //     bias[n] broadcast over rows and added after the K loop;
-//   benchmarks/silu/silu_gpu.mlir.in:3-19 for the activation fused below.
+//   benchmarks/silu/silu_gpu.mlir.in:3-19 for the activation fused below;
+//   test/Integration/Dialect/XeGPU/WG/gemm_4kx4kx4k_transpose_{a,b}.mlir for the
+//     operand storage orders (the same kernel with the other operand loader).
 //
 // Blocking on MI355X:
 //   workgroup tile 256 x 256, 512 threads = 8 wavefronts in a 2 x 4 grid (two per
