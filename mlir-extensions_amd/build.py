@@ -27,7 +27,7 @@ INCLUDE_DIR = os.path.join(REPO_DIR, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
-KERNEL_GROUPS = ["eltwise", "softmax", "reduce", "transpose", "gemm", "fusion", "attention"]
+KERNEL_GROUPS = ["eltwise", "softmax", "reduce", "transpose", "gemm", "fusion", "attention", "probe"]
 
 # -ffp-contract=off: the SiLU, scalar-GEMM and reduction kernels rely on
 # separately rounded multiplies and adds.  Packed-FP32 instruction selection is

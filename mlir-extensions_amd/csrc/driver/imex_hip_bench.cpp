@@ -108,6 +108,12 @@ std::vector<Workload> workloads() {
        {{Elem::F16, {16 * K4, 64}, true, -1, 1}, {Elem::F16, {16 * K4, 64}, true, -1, 1},
         {Elem::F16, {16 * K4, 64}, true, -1, 1}, {Elem::F16, {16 * K4, 64}, false, 0, 0}},
        {16, K4}, 2, 4.0 * 16 * K4 * K4 * 64, true},
+      // not operators: the MFMA pipe fed from LDS with nothing else going on, one workgroup per CU,
+      // on hashed f16 operands in (-1,1) and on zeros -- the rate the GEMMs' operand values allow
+      {"mfma_lds_ceiling_f16_random", "imex_mfma_lds_ceiling_f16", {256 * 512},
+       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 4096, 0}, 0, 256.0 * 8 * 4096 * 8 * 32768, true},
+      {"mfma_lds_ceiling_f16_zeros", "imex_mfma_lds_ceiling_f16", {256 * 512},
+       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 4096, 1}, 0, 256.0 * 8 * 4096 * 8 * 32768, true},
   };
 }
 

@@ -1,0 +1,86 @@
+//===- probe.hip - what the MFMA pipe sustains on given operand values ------===//
+//
+// A measurement kernel, not an operator (no counterpart in the reference): the
+// inner product loop of the tiled GEMM with everything but the matrix pipe and
+// its LDS operand reads taken away -- no global loads, no barriers in the loop,
+// no epilogue beyond one store per lane.
+//
+// Why it exists: on MI355X the shader clock under MFMA load depends on the
+// operand VALUES (switching activity in the multiplier arrays).  With f16
+// operands drawn uniformly from (-1, 1) the part settles well below the clock
+// its 2.5 PFLOP/s peak is quoted at; with all-zero operands it does not.  This
+// kernel measures that ceiling directly, on the same kind of data the GEMM
+// benchmark uses, so the GEMM's rate can be held against what the silicon
+// sustains on that data as well as against the published peak.
+//
+//   imex_mfma_lds_ceiling_f16(out: f32*, outCount: i64, iters: i64, zero: i64)
+//
+// Each workgroup (512 lanes = 8 wavefronts, two per SIMD, like the GEMM) fills
+// 64 KiB of LDS with hashed f16 pairs in (-1, 1) -- or zeros if `zero` != 0 --
+// and then runs `iters` steps of: 4 A fragments + 2 B fragments read from LDS
+// with ds_read_b128 at a position that moves every step, 8 MFMA 32x32x16 on
+// them.  FLOP per launch = gridX * 8 * iters * 8 * 2*32*32*16.  One f32 per
+// lane is stored at the end (guarded by outCount) so the work is observable.
+//
+//===----------------------------------------------------------------------===//
+
+#include "device_common.h"
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 512;
+constexpr int kLdsBytes = 65536;
+constexpr int kSlots = kLdsBytes / 16; // 16-byte operand slots
+constexpr int kFragsA = 4, kFragsB = 2;
+
+} // namespace
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_mfma_lds_ceiling_f16(float *out, int64_t outCount,
+                                                                                  int64_t iters, int64_t zero) {
+  __shared__ __attribute__((aligned(16))) uint32_t lds[kLdsBytes / 4];
+  for (int i = threadIdx.x; i < kLdsBytes / 4; i += kThreads) {
+    uint32_t x = (static_cast<uint32_t>(i) + blockIdx.x * 7919u) * 2654435761u;
+    x ^= x >> 15;
+    x *= 2246822519u;
+    x ^= x >> 13;
+    // two f16 values: random sign and mantissa, exponent field 0..14, i.e. |v| < 1
+    const uint32_t lo = (x & 0x83ffu) | (((x >> 10) % 15u) << 10);
+    const uint32_t hi = ((x >> 16) & 0x83ffu) | (((x >> 26) % 15u) << 10);
+    lds[i] = zero ? 0u : (lo | (hi << 16));
+  }
+  __syncthreads();
+
+  f32x16 acc[kFragsA * kFragsB];
+  for (int i = 0; i < kFragsA * kFragsB; ++i)
+    for (int r = 0; r < 16; ++r)
+      acc[i][r] = 0.0f;
+
+  const f16x8 *slots = reinterpret_cast<const f16x8 *>(lds);
+  const int lane = threadIdx.x;
+  for (int64_t it = 0; it < iters; ++it) {
+    const int off = static_cast<int>(it & 63) * 64;
+    f16x8 a[kFragsA], b[kFragsB];
+#pragma unroll
+    for (int i = 0; i < kFragsA; ++i)
+      a[i] = slots[(lane + off + i * 512) & (kSlots - 1)];
+#pragma unroll
+    for (int j = 0; j < kFragsB; ++j)
+      b[j] = slots[(lane + off + 2048 + j * 512) & (kSlots - 1)];
+#pragma unroll
+    for (int i = 0; i < kFragsA; ++i)
+#pragma unroll
+      for (int j = 0; j < kFragsB; ++j)
+        acc[i * kFragsB + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i * kFragsB + j], 0, 0, 0);
+  }
+
+  float s = 0.0f;
+  for (int i = 0; i < kFragsA * kFragsB; ++i)
+    for (int r = 0; r < 16; ++r)
+      s += acc[i][r];
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx < outCount)
+    out[idx] = s;
+}

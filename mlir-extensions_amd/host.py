@@ -385,6 +385,19 @@ def flash_attention(stream, q, k, v, zh, n_ctx, sm_scale):
             stream.free(p)
 
 
+def mfma_lds_ceiling(stream, workgroups, iters, zero=False):
+    """The measurement kernel imex_mfma_lds_ceiling_f16 (no counterpart in the reference):
+    returns the one f32 per lane it stores, shape (workgroups, 512)."""
+    n = workgroups * 512
+    d_o = stream.alloc(max(n, 1) * 4)
+    try:
+        stream.launch("imex_mfma_lds_ceiling_f16", [n], [d_o, n, int(iters), 1 if zero else 0])
+        stream.wait()
+        return stream.from_device(d_o, (workgroups, 512), np.float32)
+    finally:
+        stream.free(d_o)
+
+
 def softmax(stream, x, dtype="f32"):
     """benchmarks/softmax/softmax_gpu.mlir.in:4-44 (last dim of a 2-D tensor)"""
     rows, cols = x.shape

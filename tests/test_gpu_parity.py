@@ -586,3 +586,54 @@ def test_gemm_f16_output_variant(host, orc, stream):
     got = orc.half_to_float(host.gemm(stream, a, b, ab_dtype="f16", out_dtype="f16"))
     ref = orc.gemm(a, b, "f16", out_round="f16")
     assert gemm_close(got, ref)
+
+
+# ==================== MFMA ceiling measurement kernel ======================
+def _ceiling_lds_f16(workgroup):
+    """The f16 operands imex_mfma_lds_ceiling_f16 writes into LDS, as (4096 slots, 8)."""
+    with np.errstate(over="ignore"):
+        i = np.arange(16384, dtype=np.uint32)
+        x = (i + np.uint32(workgroup * 7919)) * np.uint32(2654435761)
+        x ^= x >> np.uint32(15)
+        x *= np.uint32(2246822519)
+        x ^= x >> np.uint32(13)
+    lo = (x & np.uint32(0x83ff)) | (((x >> np.uint32(10)) % np.uint32(15)) << np.uint32(10))
+    hi = ((x >> np.uint32(16)) & np.uint32(0x83ff)) | (((x >> np.uint32(26)) % np.uint32(15)) << np.uint32(10))
+    words = lo | (hi << np.uint32(16))
+    return words.view(np.uint16).view(np.float16).astype(np.float64).reshape(4096, 8)
+
+
+def test_mfma_ceiling_kernel_computes_what_it_says(host, stream):
+    """No oracle and no reference counterpart: the expected sums follow from the published
+    operand / accumulator lane layout of MFMA 32x32x16 (A[m = l%32][k = 8(l/32)..+8],
+    B likewise in n, C[8(r/4) + 4(l/32) + r%4][l%32] in register r), in f64."""
+    iters, groups = 5, 3
+    say("mfma ceiling probe: %d workgroups x %d steps" % (groups, iters))
+    got = host.mfma_lds_ceiling(stream, groups, iters)
+    assert got.shape == (groups, 512)
+    l = np.arange(64)
+    rows = (8 * (np.arange(16)[None, :] // 4) + 4 * (l[:, None] // 32) + np.arange(16)[None, :] % 4)  # [lane, r]
+    for g in range(groups):
+        slots = _ceiling_lds_f16(g)
+        for w in range(8):
+            lane = w * 64 + l
+            total = np.zeros(64)
+            for it in range(iters):
+                off = (it & 63) * 64
+                frag = lambda base: slots[(lane + off + base) & 4095]          # [64 lanes, 8 k]
+                def tile(f):                                                     # -> [32, 16]
+                    t = np.zeros((32, 16))
+                    for k8 in range(2):
+                        t[:, 8 * k8:8 * k8 + 8] = f[32 * k8:32 * k8 + 32]
+                    return t
+                for i in range(4):
+                    A = tile(frag(i * 512))
+                    for j in range(2):
+                        Bt = tile(frag(2048 + j * 512))                          # [n, k]
+                        Cm = A @ Bt.T
+                        total += Cm[rows, (l % 32)[:, None]].sum(axis=1)
+            want = total
+            have = got[g, w * 64:(w + 1) * 64].astype(np.float64)
+            assert np.all(np.abs(have - want) <= 1e-4 * np.abs(want).max() + 1e-4), (g, w)
+    assert not np.any(host.mfma_lds_ceiling(stream, 2, 7, zero=True))
+    assert host.mfma_lds_ceiling(stream, 1, 0).shape == (1, 512) and not np.any(host.mfma_lds_ceiling(stream, 1, 0))

@@ -88,6 +88,8 @@ def test_launch_shapes(host):
     assert ls("imex_input_fusion_f32", [512, 1024])[0] == (4, 1, 1)
     assert ls("imex_gemm_4kx4kx4k_transpose_a", []) == ((16, 16, 1), (512, 1, 1), 0)
     assert ls("imex_gemm_f16_f16_f32_tb", [512, 256, 96])[0] == (2, 1, 1)
+    assert ls("imex_mfma_lds_ceiling_f16", [256 * 512]) == ((256, 1, 1), (512, 1, 1), 0)
+    assert ls("imex_mfma_lds_ceiling_f16", [513])[0] == (2, 1, 1)
     with pytest.raises(ValueError):
         ls("imex_relu_f32", [1, 2])
     with pytest.raises(ValueError):
