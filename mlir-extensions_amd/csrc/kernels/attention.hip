@@ -43,14 +43,10 @@ namespace {
 
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / 64;
-constexpr int kKeyGroups = kWaves / 2;  // wavefronts that split the keys of one query half
 constexpr int D = 64;                 // head dimension
-constexpr int BM = 64;                // queries per workgroup
-constexpr int BN = 64;                // keys per tile; a ring stage holds one tile per key group
+constexpr int BN = 64;                // keys per tile; a ring stage holds one K and one V tile per key group
 constexpr int kTileBytes = BN * D * 2;          // 8 KiB
-constexpr int kStageBytes = 2 * kKeyGroups * kTileBytes; // K0..K3, V0..V3 = 64 KiB
-constexpr int kStages = 2;
-constexpr int kDmaPerWave = kStageBytes / 1024 / kWaves; // 8 copies of 1 KiB per wavefront and stage
+constexpr int kLdsBytes = 128 * 1024;           // the ring: 2 stages of 64 KiB, 4 of 32 KiB or 8 of 16 KiB
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
@@ -102,16 +98,25 @@ __device__ __forceinline__ void attention_scalar(const uint16_t *Q, const uint16
 }
 
 // ---- MFMA path ---------------------------------------------------------------------------
+// QB = 32-query blocks per workgroup (2, 4 or 8); the 8 wavefronts are QB query blocks x KG = 8 / QB
+// key groups.  More query blocks mean fewer workgroups but proportionally less K / V traffic from L2
+// (every workgroup walks all keys of its head), smaller ring stages and therefore a deeper ring.
+template <int QB>
 __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K,
                                                 const uint16_t *__restrict__ V, uint16_t *__restrict__ Out,
                                                 float scale, int64_t N, char *lds) {
   LdsChar *ldsBase = (LdsChar *)lds;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wq = wave & 1, wk = wave >> 1;
+  constexpr int KG = kWaves / QB;                  // key groups: wavefronts that split the keys of one query block
+  constexpr int kStageBytes = 2 * KG * kTileBytes; // K tiles of all key groups, then their V tiles
+  constexpr int kStages = kLdsBytes / kStageBytes; // 2, 4 or 8
+  constexpr int kAhead = kStages - 1;              // blocks in flight ahead of the one being multiplied
+  constexpr int kCopies = KG;                      // 1 KiB copies per wavefront, stage and operand
+  const int wq = wave % QB, wk = wave / QB;
   const int qi = lane & 31, half = lane >> 5;
   const int64_t head0 = int64_t(blockIdx.y) * N;         // first row of this (batch, head)
-  const int64_t q0 = head0 + int64_t(blockIdx.x) * BM + wq * 32;
+  const int64_t q0 = head0 + int64_t(blockIdx.x) * (32 * QB) + wq * 32;
 
   // Q^T operand: lane (q, half) keeps Q[q][ds*16 + half*8 .. +7] for the four 16-wide steps
   f16x8 qf[4];
@@ -119,33 +124,33 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
   for (int ds = 0; ds < 4; ++ds)
     qf[ds] = *reinterpret_cast<const f16x8 *>(Q + (q0 + qi) * D + ds * 16 + half * 8);
 
-  // -- global -> LDS copies.  A stage is [K tile 0][K tile 1][V tile 0][V tile 1], each 64
+  // -- global -> LDS copies.  A stage is [K tile 0 .. KG-1][V tile 0 .. KG-1], each 64
   // rows of 128 bytes; one copy = 8 rows.  16-byte chunk c of row r is stored at
   //   K: c ^ ((r ^ (r>>3 & 3)) & 7)   (conflict-free 128-bit fragment reads; same for r and r+32)
   //   V: c ^ (((r>>1) & 1) << 2)     (conflict-free transpose reads)
   // applied on the global side, since a direct copy fixes the lane's LDS position.
   const __amdgpu_buffer_rsrc_t kRsrc = make_rsrc(K + head0 * D, N * D * 2);
   const __amdgpu_buffer_rsrc_t vRsrc = make_rsrc(V + head0 * D, N * D * 2);
-  int kVoff[4], vVoff[4];
+  int kVoff[kCopies], vVoff[kCopies];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    // wavefront w copies rows [32w, 32w+32) of the stage's 256 K rows and of its 256 V rows
-    const int row = wave * 32 + c * 8 + (lane >> 3); // 0..255: key within the 256-key stage
+  for (int c = 0; c < kCopies; ++c) {
+    // wavefront w copies rows [8 KG w, 8 KG (w+1)) of the stage's 64 KG K rows and of its V rows
+    const int row = wave * (8 * KG) + c * 8 + (lane >> 3); // key within the stage's block of 64 KG keys
     const int r = row & 63;                          // row within its tile
     const int kc = (lane & 7) ^ ((r ^ ((r >> 3) & 3)) & 7);
     const int vc = (lane & 7) ^ (((r >> 1) & 1) << 2);
     kVoff[c] = (row * D + kc * 8) * 2;
     vVoff[c] = (row * D + vc * 8) * 2;
   }
-  auto dma_stage = [&](int it, int stageOff) { // keys [256 it, 256 it + 256)
-    LdsChar *dst = ldsBase + stageOff + wave * 4096;
-    const int soff = it * (kKeyGroups * BN * D * 2);
+  auto dma_stage = [&](int block, int stage) { // keys [64 KG block, 64 KG (block + 1)) into ring stage `stage`
+    LdsChar *dst = ldsBase + stage * kStageBytes + wave * (KG * 1024);
+    const int soff = block * (KG * BN * D * 2);
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
+    for (int c = 0; c < kCopies; ++c)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(kRsrc, dst + c * 1024, 16, kVoff[c], soff, 0, 0);
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(vRsrc, dst + kKeyGroups * kTileBytes + c * 1024, 16, vVoff[c], soff, 0, 0);
+    for (int c = 0; c < kCopies; ++c)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vRsrc, dst + KG * kTileBytes + c * 1024, 16, vVoff[c], soff, 0, 0);
   };
 
   // -- LDS read addresses (relative to this wavefront's K / V tile of a stage)
@@ -167,7 +172,7 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
 #pragma unroll
     for (int db = 0; db < 2; ++db) {
       const int chunk = ((db ^ ((t >> 3) & 1)) << 2) | (blk << 1) | ((t & 3) >> 1);
-      vRd[db] = kKeyGroups * kTileBytes + wk * kTileBytes + row * 128 + chunk * 16 + (t & 1) * 8;
+      vRd[db] = KG * kTileBytes + wk * kTileBytes + row * 128 + chunk * 16 + (t & 1) * 8;
     }
   }
 
@@ -181,15 +186,19 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
   float l = 0.0f;              // running sum of p over THIS lane's keys only
   const float c = scale * 1.44269504088896341f;
 
-  const int iters = int(N / (kKeyGroups * BN));
-  dma_stage(0, 0);
-  int curOff = 0;
+  // The ring always holds kAhead blocks in flight (past the end the last block is simply fetched
+  // again, into stages nobody reads any more), so "block `it` has landed" is one fixed vmcnt.
+  const int iters = int(N / (KG * BN));
+#pragma unroll
+  for (int b = 0; b < kAhead; ++b)
+    dma_stage(min(b, iters - 1), b);
+  int cur = 0; // ring stage of block `it`
   for (int it = 0; it < iters; ++it) {
-    wait_vmcnt<0>();              // block `it` has landed (this wavefront's copies)
-    __builtin_amdgcn_s_barrier(); // ... everyone's; and everyone is done reading block it-1
+    wait_vmcnt<(kAhead - 1) * 2 * kCopies>(); // block `it` has landed (this wavefront's copies)
+    __builtin_amdgcn_s_barrier();             // ... everyone's; and everyone is done reading block it-1
     __builtin_amdgcn_sched_barrier(0);
-    dma_stage(min(it + 1, iters - 1), curOff ^ kStageBytes); // into the stage block it-1 occupied
-    const char *st = lds + curOff;
+    dma_stage(min(it + kAhead, iters - 1), cur == 0 ? kStages - 1 : cur - 1); // into the stage block it-1 occupied
+    const char *st = lds + cur * kStageBytes;
 
     // S^T = K . Q^T for this wavefront's 64 keys (the first product of each chain takes a
     // literal zero accumulator, so no registers are cleared)
@@ -251,7 +260,7 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
         o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[kk], o[db], 0, 0, 0);
       }
     }
-    curOff ^= kStageBytes;
+    cur = cur == kStages - 1 ? 0 : cur + 1;
   }
   wait_vmcnt<0>();
   l += other_half(l); // both key halves of the lane pair
@@ -259,7 +268,7 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
   // -- merge the key groups through LDS: groups 1.. hand (m, l, O^T) to group 0
   __syncthreads(); // the ring is free
   constexpr int kSlot = 34 * 64; // floats per (query half, key group): 32 accumulator rows, m, l
-  float *xchg = reinterpret_cast<float *>(lds) + wq * (kKeyGroups - 1) * kSlot;
+  float *xchg = reinterpret_cast<float *>(lds) + wq * (KG - 1) * kSlot;
   if (wk != 0) {
     float *mine = xchg + (wk - 1) * kSlot;
 #pragma unroll
@@ -274,13 +283,13 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
   if (wk == 0) {
     float mAll = m;
 #pragma unroll
-    for (int g = 0; g < kKeyGroups - 1; ++g)
+    for (int g = 0; g < KG - 1; ++g)
       mAll = fmaxf(mAll, xchg[g * kSlot + 32 * 64 + lane]);
-    float a[kKeyGroups];
+    float a[KG];
     a[0] = exp2f(m - mAll);
     float lAll = l * a[0];
 #pragma unroll
-    for (int g = 0; g < kKeyGroups - 1; ++g) {
+    for (int g = 0; g < KG - 1; ++g) {
       a[g + 1] = exp2f(xchg[g * kSlot + 32 * 64 + lane] - mAll);
       lAll += xchg[g * kSlot + 33 * 64 + lane] * a[g + 1];
     }
@@ -296,7 +305,7 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
           const int r = g4 * 4 + e;
           float acc = o[db][r] * a[0];
 #pragma unroll
-          for (int g = 0; g < kKeyGroups - 1; ++g)
+          for (int g = 0; g < KG - 1; ++g)
             acc += xchg[g * kSlot + (db * 16 + r) * 64 + lane] * a[g + 1];
           out4[e] = static_cast<_Float16>(acc * inv);
         }
@@ -312,13 +321,17 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_flash_attention_fwd_
                                                                                    const uint16_t *V,
                                                                                    uint16_t *Out, float sm_scale,
                                                                                    int64_t ZH, int64_t N_CTX) {
-  __shared__ __attribute__((aligned(16))) char lds[kStages * kStageBytes];
-  const bool tileable = N_CTX > 0 && N_CTX % (kKeyGroups * BN) == 0 && gridDim.x == N_CTX / BM && gridDim.y == ZH &&
-                        gridDim.z == 1 &&
-                        ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
-                          reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(Out)) & 15) == 0;
-  if (tileable)
-    attention_tiled(Q, K, V, Out, sm_scale, N_CTX, lds);
+  __shared__ __attribute__((aligned(16))) char lds[kLdsBytes];
+  // The grid says how many queries a workgroup takes: N_CTX / gridDim.x = 64, 128 or 256.
+  const bool shaped = N_CTX > 0 && N_CTX % 256 == 0 && gridDim.y == ZH && gridDim.z == 1 &&
+                      ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
+                        reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(Out)) & 15) == 0;
+  if (shaped && int64_t(gridDim.x) * 64 == N_CTX)
+    attention_tiled<2>(Q, K, V, Out, sm_scale, N_CTX, lds);
+  else if (shaped && int64_t(gridDim.x) * 128 == N_CTX)
+    attention_tiled<4>(Q, K, V, Out, sm_scale, N_CTX, lds);
+  else if (shaped && int64_t(gridDim.x) * 256 == N_CTX)
+    attention_tiled<8>(Q, K, V, Out, sm_scale, N_CTX, lds);
   else
     attention_scalar(Q, K, V, Out, sm_scale, ZH, N_CTX);
 }

@@ -195,11 +195,17 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
       grid[2] = 65535;
     break;
   }
-  case Shape::Attention: { // dims = {ZH, N_CTX}; 64 queries x 8 wavefronts per workgroup when N_CTX % 256 == 0
+  case Shape::Attention: {
+    // dims = {ZH, N_CTX}.  When N_CTX % 256 == 0 a workgroup (8 wavefronts) takes 64, 128 or 256 queries of
+    // one (batch, head); the kernel reads the choice off the grid.  More queries per workgroup mean less
+    // K / V traffic, so: the largest of the three that still gives every one of the 256 CUs a workgroup.
     const int64_t ZH = dims[0], N = dims[1];
     block[0] = 512;
     if (N > 0 && N % 256 == 0 && ZH > 0 && ZH <= 65535) {
-      grid[0] = static_cast<size_t>(N / 64);
+      int64_t queries = 256;
+      while (queries > 64 && (N / queries) * ZH < 256)
+        queries /= 2;
+      grid[0] = static_cast<size_t>(N / queries);
       grid[1] = static_cast<size_t>(ZH);
     } else {
       grid[0] = ceilDiv(ZH * N, 512); // one lane per query

@@ -351,6 +351,37 @@ def test_flash_attention_sixteen_heads(host, orc, stream):
     assert attention_close(got[rows], orc.flash_attention_rows(q, k, v, n_ctx, scale, rows), orc)
 
 
+@pytest.mark.parametrize("zh,n_ctx,scale", [(3, 512, 0.5), (2, 256, 4.0), (1, 2048, 0.125)])
+def test_flash_attention_every_tiling(host, orc, stream, zh, n_ctx, scale):
+    """64, 128 and 256 queries per workgroup (2, 4, 8 query blocks x 4, 2, 1 key groups; ring of
+    2, 4, 8 stages): each against the oracle, on the same inputs."""
+    n = zh * n_ctx
+    q = orc.fill_uniform(n * 64, "f16", 71, -2, 2).reshape(n, 64)
+    k = orc.fill_uniform(n * 64, "f16", 72, -2, 2).reshape(n, 64)
+    v = orc.fill_uniform(n * 64, "f16", 73, -1, 1).reshape(n, 64)
+    rows = np.unique(np.concatenate([np.arange(0, n, 7), [n_ctx - 1, n - 1]]))
+    ref = orc.flash_attention_rows(q, k, v, n_ctx, scale, rows)
+    for queries in (64, 128, 256):
+        say("attention %dx%d, %d queries per workgroup" % (zh, n_ctx, queries))
+        got = host.flash_attention(stream, q, k, v, zh, n_ctx, scale, queries_per_workgroup=queries)
+        assert attention_close(got[rows], ref, orc), queries
+
+
+@pytest.mark.parametrize("zh", [8, 16])
+def test_flash_attention_catalogue_picks_wide_tilings(host, orc, stream, zh):
+    """N_CTX = 4096 with 8 and 16 heads: the catalogue launches 128- and 256-query workgroups
+    (16 heads is the reference's flash_attention_fwd_ov_with_arrray_len_4k.mlir shape)."""
+    n_ctx = 4096
+    assert host.launch_shape("imex_flash_attention_fwd_f16", [zh, n_ctx])[0] == (n_ctx // (16 * zh), zh, 1)
+    n = zh * n_ctx
+    q = orc.fill_uniform(n * 64, "f16", 74, -1, 1).reshape(n, 64)
+    k = orc.fill_uniform(n * 64, "f16", 75, -1, 1).reshape(n, 64)
+    v = orc.fill_uniform(n * 64, "f16", 76, -1, 1).reshape(n, 64)
+    got = host.flash_attention(stream, q, k, v, zh, n_ctx, 0.5)
+    rows = np.unique(np.concatenate([np.arange(0, n, 2999), [255, 256, n_ctx - 1, n_ctx, n - 1]]))
+    assert attention_close(got[rows], orc.flash_attention_rows(q, k, v, n_ctx, 0.5, rows), orc)
+
+
 def test_flash_attention_sharp_scores(host, orc, stream):
     """Large score range (scale 4, |q.k| up to ~20): the running max changes from block
     to block and the rescaling of the accumulator is exercised."""
