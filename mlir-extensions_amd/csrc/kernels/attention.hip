@@ -115,8 +115,20 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
   constexpr int kCopies = KG;                      // 1 KiB copies per wavefront, stage and operand
   const int wq = wave % QB, wk = wave / QB;
   const int qi = lane & 31, half = lane >> 5;
-  const int64_t head0 = int64_t(blockIdx.y) * N;         // first row of this (batch, head)
-  const int64_t q0 = head0 + int64_t(blockIdx.x) * (32 * QB) + wq * 32;
+  // Workgroups go to the 8 XCDs round-robin in launch order, and each XCD has its own L2.  Renumber
+  // them so that one XCD gets consecutive query blocks -- whole heads, or a contiguous part of one --
+  // and its L2 holds the K / V of a few heads instead of a slice of the traffic of all of them.
+  uint32_t bx = blockIdx.x, by = blockIdx.y;
+  {
+    const uint32_t total = gridDim.x * gridDim.y, launched = by * gridDim.x + bx;
+    if (total % 8 == 0) {
+      const uint32_t logical = (launched & 7) * (total >> 3) + (launched >> 3);
+      by = logical / gridDim.x;
+      bx = logical - by * gridDim.x;
+    }
+  }
+  const int64_t head0 = int64_t(by) * N;                 // first row of this (batch, head)
+  const int64_t q0 = head0 + int64_t(bx) * (32 * QB) + wq * 32;
 
   // Q^T operand: lane (q, half) keeps Q[q][ds*16 + half*8 .. +7] for the four 16-wide steps
   f16x8 qf[4];
