@@ -21,19 +21,20 @@
 // plain register loops plus ONE exchange between lane l and l+32 per block of
 // keys.
 //
-// Workgroup = 64 queries of one (batch, head): 8 wavefronts = 2 query halves x 4
-// key groups (wavefront w takes queries 32*(w&1).. and every fourth 64-key tile,
-// group w>>1), partial (m, l, O) of the four groups merged through LDS at the
-// end.  That keeps 256 workgroups in flight for the reference's shape
-// (2 x 2 x 4096 x 64: one per CU) where a 128-query tile would fill half the
-// chip, and puts two wavefronts on every SIMD, so one's MFMAs run under the
-// other's exponentials.  K and V blocks of 256 keys go from global memory straight
-// into a two-stage LDS ring (buffer_load ... lds), one block ahead.
+// Workgroup = 8 wavefronts = QB query blocks of 32 x 8/QB key groups, i.e. 64, 128 or 256
+// queries of one (batch, head) (QB = 2, 4, 8; wavefront w takes query block w % QB and every
+// (8/QB)-th 64-key tile, group w / QB); partial (m, l, O) of the key groups are merged through
+// LDS at the end.  Every workgroup walks all keys of its head, so K / V traffic from L2 falls
+// with the queries per workgroup; key groups exist to keep all CUs busy on small problems (the
+// reference's 2 x 2 x 4096 x 64 gives one 64-query workgroup per CU).  The grid says which: the
+// kernel takes N_CTX / gridDim.x queries per workgroup.  Two wavefronts share each SIMD.  K and
+// V blocks of 64 * 8/QB keys go from global memory straight into an LDS ring (buffer_load ...
+// lds) of 2, 4 or 8 stages, up to seven blocks ahead.
 //
 // Arguments: (Q, K, V, Out, sm_scale: f32, ZH: i64, N_CTX: i64)   dims = {ZH, N_CTX}
 //   ZH = batch * heads; N_CTX a multiple of 256; all four tensors [(ZH*N_CTX), 64].
-// Launch: block (512,1,1); grid (N_CTX/64, ZH, 1).  Other shapes take the
-// one-query-per-lane reference loop of the same kernel (grid-stride, any grid).
+// Launch: block (512,1,1); grid (N_CTX / q, ZH, 1) with q = 64, 128 or 256.  Other shapes and
+// grids take the one-query-per-lane reference loop of the same kernel (grid-stride, any grid).
 
 #include "device_common.h"
 
