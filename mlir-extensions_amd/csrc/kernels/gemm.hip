@@ -34,12 +34,15 @@
 //   (ids congruent mod 8) cover a compact 4 x 8 block of tiles and share A and
 //   B panels in that XCD's L2.
 //
-// Shapes that are not multiples of the tile (M%256, N%256, K%32) take the
-// one-thread-per-output path of the same kernels, which adds in ascending k
-// like the reference's CPU loop (lib/ExecutionEngine/ImexRunnerUtils.cpp:308-317).
+// M and N need not divide the tile: edge tiles copy the last row / column that exists
+// in place of the missing ones and store only what is inside C.  What the MFMA path
+// does need is K in whole steps of 32 and 16-byte aligned rows in memory (N % 8 == 0
+// where B is [K,N], M % 8 == 0 where A is [K,M]); other shapes take the
+// one-thread-per-output path of the same kernels, which adds in ascending k like the
+// reference's CPU loop (lib/ExecutionEngine/ImexRunnerUtils.cpp:308-317).
 //
-// Launch: block (512,1,1); grid (tiles,1,1) with tiles = (M/256)*(N/256) when
-// the shape is tileable, else (ceil(M*N/512),1,1).  The fixed-shape 4096^3 entry
+// Launch: block (512,1,1); grid (tiles,1,1) with tiles = ceil(M/256)*ceil(N/256) on
+// the MFMA path, else (ceil(M*N/512),1,1).  The fixed-shape 4096^3 entry
 // points take the reference's own launch: blocks (16,16,1), threads (512,1,1).
 
 #include "device_common.h"
@@ -184,15 +187,20 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
 
   // ptr: the operand's matrix; ld: its leading dimension; first: first row (m0 or n0)
   // of the slab; w0: the wavefront's first row inside the slab; extent: rows * cols.
+  // A slab that sticks out of the matrix (last tile row / column of a ragged shape): the
+  // lanes that would copy rows past the end copy the last row that exists instead, so no
+  // address ever leaves the matrix; those rows only feed outputs that are never stored.
   __device__ __forceinline__ void setup(const uint16_t *ptr, int64_t ld, int64_t first, int w0, int64_t extent,
                                         int wave, int lane) {
     if constexpr (!kStrided) {
-      rsrc = make_rsrc(ptr + first * ld, 256 * ld * 2);
+      const int64_t rows = extent / ld - first; // rows of the matrix from `first` on, >= 1
+      const int last = rows < 256 ? int(rows) - 1 : 255;
+      rsrc = make_rsrc(ptr + first * ld, int64_t(last + 1) * ld * 2);
 #pragma unroll
       for (int q = 0; q < kDmaPerWave; ++q) {
         const int row = wave * (256 / kWaves) + q * 16 + (lane >> 2);
         const int chunk = (lane & 3) ^ ((row >> 2) & 3);
-        voff[q] = int((int64_t(row) * ld + chunk * 8) * 2);
+        voff[q] = int((int64_t(min(row, last)) * ld + chunk * 8) * 2);
       }
       step = RK * 2;
       dstWave = wave * (256 / kWaves) * (RK * 2);
@@ -207,7 +215,8 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
         const int row = wave * (RK / kWaves) + q * 2 + (lane >> 5);
         const int g = (row & 3) | (((row >> 3) & 1) << 2);
         const int chunk = (((((lane & 31) >> 1) ^ g)) << 1) | (lane & 1);
-        voff[q] = int((int64_t(row) * ld + chunk * 8) * 2);
+        const int64_t col = min(int64_t(chunk * 8), ld - 8 - first); // ld % 8 == 0: the last 16 bytes of the k-row
+        voff[q] = int((int64_t(row) * ld + col) * 2);
       }
       step = int(RK * ld * 2);
       dstWave = wave * (RK / kWaves) * 512;
@@ -251,7 +260,7 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
   const int wm = wave / kWavesN, wn = wave % kWavesN;
 
   // -- workgroup id -> tile, XCD-aware ------------------------------------------------
-  const int tilesM = int(M / BM), tilesN = int(N / BN);
+  const int tilesM = int((M + BM - 1) / BM), tilesN = int((N + BN - 1) / BN);
   const int tiles = tilesM * tilesN;
   int pid = blockIdx.y * gridDim.x + blockIdx.x;
   if (pid >= tiles)
@@ -341,16 +350,27 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
   // -- epilogue: lane holds, for tile (i,j), column n = lane%32 and rows
   //    (r/4)*8 + (lane/32)*4 + r%4, r = 0..15.
   const int fragRow = lane & 31, fragHalf = lane >> 5;
+  const int64_t mBase = m0 + wm * WM + fragHalf * 4, nBase = n0 + wn * WN + fragRow;
+  if (m0 + BM <= M && n0 + BN <= N) { // interior tile (uniform over the workgroup): nothing to mask
 #pragma unroll
-  for (int i = 0; i < TI; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < TJ; ++j)
+      for (int j = 0; j < TJ; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t m = m0 + wm * WM + i * 32 + (r >> 2) * 8 + fragHalf * 4 + (r & 3);
-        const int64_t n = n0 + wn * WN + j * 32 + fragRow;
-        epi(m, n, N, acc[i][j][r]);
-      }
+        for (int r = 0; r < 16; ++r)
+          epi(mBase + i * 32 + (r >> 2) * 8 + (r & 3), nBase + j * 32, N, acc[i][j][r]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t m = mBase + i * 32 + (r >> 2) * 8 + (r & 3), n = nBase + j * 32;
+          if (m < M && n < N)
+            epi(m, n, N, acc[i][j][r]);
+        }
+  }
 }
 
 template <typename T, bool kAT, bool kBT, typename Epi>
@@ -358,7 +378,10 @@ __device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B,
                                            Epi epi) {
   // 4 stages x (256 + 256) rows x 32 k x 2 B = 128 KiB of the CU's 160 KiB LDS.
   __shared__ __attribute__((aligned(16))) char lds[kStages * kRStage];
-  const bool tileable = (M % BM == 0) && (N % BN == 0) && (K % RK == 0) && M > 0 && N > 0 && K > 0 &&
+  // The MFMA path wants K in whole 32-wide steps and 16-byte aligned rows in memory: a row of
+  // B [K,N] (or of A [K,M] when transposed) is N (M) elements long, so those must be multiples
+  // of 8.  M and N need not divide the tile: edge tiles multiply padding and store what exists.
+  const bool tileable = M > 0 && N > 0 && K > 0 && K % RK == 0 && (kBT || N % 8 == 0) && (!kAT || M % 8 == 0) &&
                         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
   if (tileable)
     gemm_tiled<T, kAT, kBT, Epi>(A, B, M, N, K, epi, lds);

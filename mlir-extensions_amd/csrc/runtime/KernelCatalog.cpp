@@ -28,7 +28,7 @@ extern const unsigned char imex_blob_probe[], imex_blob_probe_end[];
 namespace {
 
 enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm, Fusion, Attention, Probe };
-enum class Shape { Eltwise32, Eltwise16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmFixed4k, ColumnThreads, Attention, LanesOf512 };
+enum class Shape { Eltwise32, Eltwise16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, Attention, LanesOf512 };
 
 struct Entry {
   const char *name;
@@ -76,9 +76,9 @@ const Entry kEntries[] = {
     {"imex_gemm_bf16_bias_silu_bf16", "(A: bf16*, B: bf16*, bias: f32*, out: bf16*, M: i64, N: i64, K: i64)",
      Module::Gemm, Shape::Gemm, 3},
     {"imex_gemm_f16_f16_f32_tb", "(A: f16*, Bt: f16* [N,K], C: f32*, M: i64, N: i64, K: i64)", Module::Gemm,
-     Shape::Gemm, 3},
+     Shape::GemmTB, 3},
     {"imex_gemm_f16_f16_f32_ta", "(At: f16* [K,M], B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm,
-     Shape::Gemm, 3},
+     Shape::GemmTA, 3},
     {"imex_gemm_4kx4kx4k_f16_f16_f32", "(A: f16*, B: f16*, C: f32*)", Module::Gemm, Shape::GemmFixed4k, 0},
     {"imex_gemm_4kx4kx4k_transpose_b", "(A: f16*, Bt: f16* [N,K], C: f32*)", Module::Gemm, Shape::GemmFixed4k, 0},
     {"imex_gemm_4kx4kx4k_transpose_a", "(At: f16* [K,M], B: f16*, C: f32*)", Module::Gemm, Shape::GemmFixed4k, 0},
@@ -215,11 +215,18 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
   case Shape::ColumnThreads: // one lane per output column
     grid[0] = ceilDiv(dims[1], 256);
     break;
-  case Shape::Gemm: { // 512 lanes: eight wavefronts per 256 x 256 tile
+  case Shape::Gemm:
+  case Shape::GemmTA:
+  case Shape::GemmTB: {
+    // 512 lanes: eight wavefronts per 256 x 256 tile of C, edge tiles included.  The MFMA path
+    // needs K in steps of 32 and 16-byte aligned rows in memory, i.e. N % 8 == 0 where B is
+    // [K,N] and M % 8 == 0 where A is [K,M]; everything else is one lane per output.
     const int64_t M = dims[0], N = dims[1], K = dims[2];
-    const bool tileable = M > 0 && N > 0 && K > 0 && M % 256 == 0 && N % 256 == 0 && K % 32 == 0;
+    const bool rowsB = e->shape == Shape::GemmTB || N % 8 == 0;
+    const bool rowsA = e->shape != Shape::GemmTA || M % 8 == 0;
+    const bool tileable = M > 0 && N > 0 && K > 0 && K % 32 == 0 && rowsA && rowsB;
     block[0] = 512;
-    grid[0] = tileable ? static_cast<size_t>((M / 256) * (N / 256)) : ceilDiv(M * N, 512);
+    grid[0] = tileable ? ceilDiv(M, 256) * ceilDiv(N, 256) : ceilDiv(M * N, 512);
     break;
   }
   case Shape::LanesOf512: // dims = {outCount}: one lane per output element, 512 per workgroup

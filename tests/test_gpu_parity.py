@@ -441,8 +441,10 @@ def test_gemm_golden_3x3(host, orc, stream):
     assert np.all(orc.half_to_float(out) == g["expected_fill"])
 
 
-@pytest.mark.parametrize("M,N,K", [(5, 7, 9), (100, 36, 130), (256, 256, 16), (256, 256, 48), (255, 256, 64), (17, 300, 64)])
+@pytest.mark.parametrize("M,N,K", [(5, 7, 9), (100, 36, 130), (256, 256, 16), (256, 256, 48), (255, 252, 64), (17, 300, 64)])
 def test_gemm_untileable_shapes_bit_exact(host, orc, stream, M, N, K):
+    """K not a multiple of 32 or N not a multiple of 8: the one-lane-per-output path, which
+    accumulates in the oracle's order."""
     a = orc.fill_uniform(M * K, "f16", 1, -1, 1).reshape(M, K)
     b = orc.fill_uniform(K * N, "f16", 2, -1, 1).reshape(K, N)
     assert np.array_equal(host.gemm(stream, a, b, ab_dtype="f16"), orc.gemm(a, b, "f16"))
@@ -484,6 +486,59 @@ def test_gemm_tiled_short_k_random(host, orc, stream, dtype, M, N, K):
     a = orc.fill_uniform(M * K, dtype, 11, -1, 1).reshape(M, K)
     b = orc.fill_uniform(K * N, dtype, 12, -1, 1).reshape(K, N)
     assert gemm_close(host.gemm(stream, a, b, ab_dtype=dtype), orc.gemm(a, b, dtype))
+
+
+def _gemm_guarded(host, stream, name, sa, sb, M, N, K, extra=(), out_np=np.float32):
+    """Launch a GEMM kernel on an output buffer with 256 guard rows behind it; returns the
+    [M,N] result after checking that the guard rows kept their fill."""
+    guard = 256
+    fill = np.full((M + guard, N), 0x7fc1 if out_np == np.uint16 else np.float32(-12345.5), out_np)
+    d_a, d_b, d_c = stream.to_device(sa), stream.to_device(sb), stream.to_device(fill)
+    extras = [stream.to_device(e) for e in extra]
+    try:
+        stream.launch(name, [M, N, K], [d_a, d_b] + extras + [d_c, M, N, K])
+        stream.wait()
+        out = stream.from_device(d_c, (M + guard, N), out_np)
+    finally:
+        for p in [d_a, d_b, d_c] + extras:
+            stream.free(p)
+    assert np.array_equal(out[M:], fill[M:]), "%s wrote past row %d" % (name, M)
+    return out[:M]
+
+
+@pytest.mark.parametrize("M,N,K", [(255, 256, 64), (1, 8, 32), (300, 520, 96), (257, 264, 1024), (4000, 1000, 128),
+                                   (31, 4104, 64)])
+def test_gemm_ragged_tiles(host, orc, stream, M, N, K):
+    """M and N that do not divide the 256 x 256 tile (K % 32 == 0, N % 8 == 0): the MFMA path with
+    edge tiles.  Integer operands give the exact product in any order; random ones the 5e-3 bar;
+    nothing is stored outside C."""
+    say("gemm ragged %dx%dx%d" % (M, N, K))
+    a = orc.fill_int(M * K, "f16", 5, -4, 4).reshape(M, K)
+    b = orc.fill_int(K * N, "f16", 6, -4, 4).reshape(K, N)
+    want = orc.to_float(a, "f16").astype(np.int64) @ orc.to_float(b, "f16").astype(np.int64)
+    got = _gemm_guarded(host, stream, "imex_gemm_f16_f16_f32", a, b, M, N, K)
+    assert np.array_equal(got.astype(np.int64), want)
+    a = orc.fill_uniform(M * K, "bf16", 13, -1, 1).reshape(M, K)
+    b = orc.fill_uniform(K * N, "bf16", 14, -1, 1).reshape(K, N)
+    rows = np.unique(np.concatenate([np.arange(0, M, 61), [M - 1]]))
+    got = _gemm_guarded(host, stream, "imex_gemm_bf16_bf16_f32", a, b, M, N, K)
+    assert gemm_close(got[rows], orc.gemm_rows(a, b, rows, "bf16"))
+    # fused bias + SiLU epilogue and the f16-output one on the same ragged shape
+    bias = orc.fill_normal(N, "f32", 15, 0.0, 0.1)
+    fused = _gemm_guarded(host, stream, "imex_gemm_bf16_bias_silu_bf16", a, b, M, N, K, extra=(bias,), out_np=np.uint16)
+    ref = orc.bfloat_to_float(orc.bias_silu_bf16(orc.gemm_rows(a, b, rows, "bf16"), bias))
+    assert np.max(np.abs(orc.bfloat_to_float(fused)[rows] - ref)) <= 5e-3 * np.max(np.abs(ref)) + 2.0 ** -9
+
+
+@pytest.mark.parametrize("which,M,N,K", [("ta", 248, 264, 64), ("ta", 8, 8, 32), ("tb", 100, 37, 64), ("tb", 300, 515, 96)])
+def test_gemm_ragged_tiles_transposed_operands(host, orc, stream, which, M, N, K):
+    """Edge tiles with A stored [K,M] (M % 8 == 0) or B stored [N,K] (any N)."""
+    a = orc.fill_int(M * K, "f16", 33, -4, 4).reshape(M, K)
+    b = orc.fill_int(K * N, "f16", 34, -4, 4).reshape(K, N)
+    sa, sb = (np.ascontiguousarray(a.T), b) if which == "ta" else (a, np.ascontiguousarray(b.T))
+    want = orc.to_float(a, "f16").astype(np.int64) @ orc.to_float(b, "f16").astype(np.int64)
+    got = _gemm_guarded(host, stream, "imex_gemm_f16_f16_f32_" + which, sa, sb, M, N, K)
+    assert np.array_equal(got.astype(np.int64), want)
 
 
 def test_gemm_launch_shape_slack(host, orc, stream):

@@ -77,11 +77,17 @@ def test_launch_shapes(host):
     assert ls("imex_gemm_f16_f16_f32", [4096, 4096, 4096]) == ((256, 1, 1), (512, 1, 1), 0)
     assert ls("imex_gemm_bf16_bias_silu_bf16", [4096, 11008, 4096])[0] == (16 * 43, 1, 1)
     assert ls("imex_gemm_f16_f16_f32", [3, 3, 3])[0] == (1, 1, 1)
-    # the tiled path takes K in steps of 32: the catalogue must count tiles exactly when the kernel tiles
+    # the MFMA path takes K in steps of 32 and B rows of whole 16-byte groups (N % 8 == 0); M and N need
+    # not divide the 256 x 256 tile.  The catalogue must count tiles exactly when the kernel tiles.
     assert ls("imex_gemm_f16_f16_f32", [256, 256, 32])[0] == (1, 1, 1)
     assert ls("imex_gemm_f16_f16_f32", [512, 256, 96])[0] == (2, 1, 1)
-    assert ls("imex_gemm_f16_f16_f32", [256, 256, 48])[0] == (128, 1, 1)
-    assert ls("imex_gemm_f16_f16_f32", [255, 256, 64])[0] == (128, 1, 1)
+    assert ls("imex_gemm_f16_f16_f32", [255, 256, 64])[0] == (1, 1, 1)
+    assert ls("imex_gemm_f16_f16_f32", [257, 520, 64])[0] == (6, 1, 1)
+    assert ls("imex_gemm_f16_f16_f32", [256, 256, 48])[0] == (128, 1, 1)   # K % 32 != 0: one lane per output
+    assert ls("imex_gemm_f16_f16_f32", [256, 252, 64])[0] == (126, 1, 1)   # N % 8 != 0
+    assert ls("imex_gemm_f16_f16_f32_tb", [256, 252, 64])[0] == (1, 1, 1)  # B stored [N,K]: any N
+    assert ls("imex_gemm_f16_f16_f32_ta", [252, 256, 64])[0] == (126, 1, 1)  # A stored [K,M]: M % 8 != 0
+    assert ls("imex_gemm_f16_f16_f32_ta", [248, 256, 64])[0] == (1, 1, 1)
     assert ls("imex_gemm_4kx4kx4k_f16_f16_f32", []) == ((16, 16, 1), (512, 1, 1), 0)
     assert ls("imex_flash_attention_fwd_f16", [4, 4096]) == ((64, 4, 1), (512, 1, 1), 0)
     assert ls("imex_flash_attention_fwd_f16", [2, 100])[0] == (1, 1, 1)
@@ -299,14 +305,17 @@ def test_launch_shapes_cover_the_problem(host):
         assert gx >= 1 and (gx * 4 >= rows if cols <= 1024 else gx >= min(rows, 1048560))
 
     @settings(max_examples=300, deadline=None)
-    @given(m=st.integers(1, 64), n=st.integers(1, 64), k=st.integers(1, 512), ragged=st.booleans())
-    def gemm(m, n, k, ragged):
-        M, N, K = (m * 256, n * 256, k * 32) if not ragged else (m * 37 + 1, n * 41 + 3, k * 7 + 5)
-        for name in ("imex_gemm_f16_f16_f32", "imex_gemm_f16_f16_f32_ta", "imex_gemm_bf16_bias_silu_bf16"):
+    @given(M=st.integers(1, 20000), N=st.integers(1, 20000), k=st.integers(1, 512), round_n=st.booleans(),
+           round_k=st.booleans())
+    def gemm(M, N, k, round_n, round_k):
+        N = (N + 7) // 8 * 8 if round_n else N
+        K = k * 32 if round_k else k * 7 + 5
+        for name in ("imex_gemm_f16_f16_f32", "imex_gemm_f16_f16_f32_ta", "imex_gemm_f16_f16_f32_tb",
+                     "imex_gemm_bf16_bias_silu_bf16"):
             (gx, gy, gz), block, _ = ls(name, [M, N, K])
             assert block == (512, 1, 1) and gy == gz == 1
-            tileable = M % 256 == 0 and N % 256 == 0 and K % 32 == 0
-            assert gx == (M // 256) * (N // 256) if tileable else gx * 512 >= M * N
+            tileable = K % 32 == 0 and (name.endswith("_tb") or N % 8 == 0) and (not name.endswith("_ta") or M % 8 == 0)
+            assert gx == -(-M // 256) * -(-N // 256) if tileable else gx * 512 >= M * N
 
     eltwise()
     rowwise()
