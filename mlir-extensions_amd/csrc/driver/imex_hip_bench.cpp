@@ -108,6 +108,22 @@ std::vector<Workload> workloads() {
        {{Elem::F16, {16 * K4, 64}, true, -1, 1}, {Elem::F16, {16 * K4, 64}, true, -1, 1},
         {Elem::F16, {16 * K4, 64}, true, -1, 1}, {Elem::F16, {16 * K4, 64}, false, 0, 0}},
        {16, K4}, 2, 4.0 * 16 * K4 * K4 * 64, true},
+      // shapes of the reference's benchmark suite (README.md:330-335) beyond the ones above
+      {"relu_f32_512x640x20x15", "imex_relu_f32", {98304000},
+       {{Elem::F32, {98304000}, true, -1, 1}, {Elem::F32, {98304000}, false, 0, 0}}, {98304000}, 0,
+       2.0 * 98304000 * 4, false},
+      {"reduce_outer_f32_32x16x512x512", "imex_reduce_outer_f32", {32, 16 * 512 * 512},
+       {{Elem::F32, {32, 16 * 512 * 512}, true, 0, 1}, {Elem::F32, {16 * 512 * 512}, false, 0, 0}},
+       {32, 16 * 512 * 512}, 1, 33.0 * 16 * 512 * 512 * 4, false},
+      {"softmax_f32_1024x2000", "imex_softmax_f32", {1024, 2000},
+       {{Elem::F32, {1024, 2000}, true, -4, 4}, {Elem::F32, {1024, 2000}, false, 0, 0}}, {1024, 2000}, 0,
+       2.0 * 1024 * 2000 * 4, false},
+      {"transpose_f32_1024x1024", "imex_transpose2d_b32", {1024, 1024},
+       {{Elem::F32, {1024, 1024}, true, -1, 1}, {Elem::F32, {1024, 1024}, false, 0, 0}}, {1024, 1024}, 0,
+       2.0 * 1024 * 1024 * 4, false},
+      {"transpose3d_f32_16x96x96", "imex_transpose3d_b32", {16, 96, 96},
+       {{Elem::F32, {16, 96, 96}, true, -1, 1}, {Elem::F32, {96, 96, 16}, false, 0, 0}}, {16, 96, 96}, 0,
+       2.0 * 16 * 96 * 96 * 4, false},
       // not operators: the MFMA pipe fed from LDS with nothing else going on, one workgroup per CU,
       // on hashed f16 operands in (-1,1) and on zeros -- the rate the GEMMs' operand values allow
       {"mfma_lds_ceiling_f16_random", "imex_mfma_lds_ceiling_f16", {256 * 512},

@@ -169,9 +169,12 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
   case Shape::RowSum: // workgroup per row above 2048 columns, else wavefront per row
     grid[0] = dims[1] > 2048 ? static_cast<size_t>(dims[0]) : ceilDiv(dims[0], 4);
     break;
-  case Shape::ReduceOuter: // four outputs per lane
-    grid[0] = ceilDiv(dims[1], 1024);
+  case Shape::ReduceOuter: { // 1024 v outputs per workgroup, v = 8, 4, 2, 1: the widest that leaves 512 workgroups
+    const int64_t inner = dims[1];
+    const int64_t v = inner >= 512 * 8192 ? 8 : inner >= 512 * 4096 ? 4 : inner >= 512 * 2048 ? 2 : 1;
+    grid[0] = ceilDiv(inner, 1024 * v);
     break;
+  }
   case Shape::Transpose2D32:
   case Shape::Transpose2D16:
   case Shape::Transpose3D32:

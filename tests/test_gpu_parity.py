@@ -171,11 +171,35 @@ def test_rowsum_config_8192x8192(host, orc, stream):
     assert np.max(np.abs(got - exact) / exact) < 1e-5
 
 
-@pytest.mark.parametrize("shape", [(32, 16, 64, 64), (10, 20), (7, 1023), (33, 4100), (1, 5), (3, 1, 9)])
+@pytest.mark.parametrize("shape", [(32, 16, 64, 64), (10, 20), (7, 1023), (33, 4100), (1, 5), (3, 1, 9),
+                                   (5, 512 * 2048 + 4), (3, 512 * 4096 + 1028), (2, 512 * 8192 + 8), (6, 512 * 2048 + 3)])
 def test_reduce_outer_bit_exact(host, orc, stream, shape):
+    """The last four shapes reach the 8, 16 and 32 KiB-per-slice variants with a ragged last
+    workgroup, and the one-lane-per-output path at a size where it strides."""
     x = orc.fill_uniform(int(np.prod(shape)), "f32", 77, -1.0, 1.0).reshape(shape)
     got, ref = host.reduce_outer(stream, x, init=0.25), orc.reduce_outer_f32(x, init=0.25)
     assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+
+
+def test_reduce_outer_benchmark_shape_and_any_grid(host, orc, stream):
+    """32x16x512x512 (the reference suite's reduce shape, README.md:335): integer-valued inputs
+    make the sum exact; then the same kernel on a grid of 7 workgroups, which must stride."""
+    import ctypes as C
+    outer, inner = 32, 16 * 512 * 512
+    x = orc.fill_int(outer * inner, "f32", 78, -8, 8).reshape(outer, inner)
+    got = host.reduce_outer(stream, x, init=1.0)
+    assert np.array_equal(got, 1.0 + x.sum(axis=0, dtype=np.float64).astype(np.float32))
+    small = x[:, :300000]
+    small = np.ascontiguousarray(small)
+    d_in, d_out = stream.to_device(small), stream.alloc(small.shape[1] * 4)
+    fn = stream.kernel("imex_reduce_outer_f32")
+    descs, keep = host._pack_params([d_in, d_out, outer, small.shape[1], 1.0])
+    stream.rt.gpuLaunchKernel(stream.handle, fn, 7, 1, 1, 256, 1, 1, 0, C.cast(descs, C.c_void_p), None)
+    stream.wait()
+    out = stream.from_device(d_out, (small.shape[1],), np.float32)
+    stream.free(d_in)
+    stream.free(d_out)
+    assert np.array_equal(out, 1.0 + small.sum(axis=0, dtype=np.float64).astype(np.float32))
 
 
 # =============================== Transpose =================================
