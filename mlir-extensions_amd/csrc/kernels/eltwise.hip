@@ -110,18 +110,6 @@ __device__ const uint64_t kExp2Table[32] = {
     0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
 
 __device__ __forceinline__ float expf_libm(float x, const uint64_t *table) {
-  const uint32_t ux = f2u(x);
-  const uint32_t abstop = (ux >> 20) & 0x7ffu;
-  if (abstop >= 0x42bu) { // |x| >= 88 or NaN
-    if (ux == 0xff800000u)
-      return 0.0f;
-    if (abstop >= 0x7f8u)
-      return x + x;
-    if (x > 0x1.62e42ep6f)
-      return __builtin_inff();
-    if (x < -0x1.9fe368p6f)
-      return 0.0f;
-  }
   constexpr double kInvLn2N = 0x1.71547652b82fep+0 * 32;
   constexpr double kShift = 0x1.8p+52;
   constexpr double kC0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32;
@@ -141,7 +129,15 @@ __device__ __forceinline__ float expf_libm(float x, const uint64_t *table) {
   double y = kC2 * r + 1.0;
   y = p * r2 + y;
   y = y * s;
-  return static_cast<float>(y);
+  float result = static_cast<float>(y);
+  // |x| >= 88, infinities and NaN: libm branches to these cases before the arithmetic above; here
+  // they are selects after it (whatever the arithmetic made of such an x is discarded), which
+  // keeps the instruction stream straight -- a taken branch per element costs more than the math.
+  const uint32_t ux = f2u(x);
+  const uint32_t abstop = (ux >> 20) & 0x7ffu;
+  const float big = x > 0x1.62e42ep6f ? __builtin_inff() : (x < -0x1.9fe368p6f ? 0.0f : result);
+  const float special = abstop >= 0x7f8u ? (ux == 0xff800000u ? 0.0f : x + x) : big;
+  return abstop >= 0x42bu ? special : result;
 }
 
 struct SiluF32 {
