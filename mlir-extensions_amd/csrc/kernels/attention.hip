@@ -21,20 +21,23 @@
 // plain register loops plus ONE exchange between lane l and l+32 per block of
 // keys.
 //
-// Workgroup = 8 wavefronts = QB query blocks of 32 x 8/QB key groups, i.e. 64, 128 or 256
-// queries of one (batch, head) (QB = 2, 4, 8; wavefront w takes query block w % QB and every
-// (8/QB)-th 64-key tile, group w / QB); partial (m, l, O) of the key groups are merged through
-// LDS at the end.  Every workgroup walks all keys of its head, so K / V traffic from L2 falls
-// with the queries per workgroup; key groups exist to keep all CUs busy on small problems (the
-// reference's 2 x 2 x 4096 x 64 gives one 64-query workgroup per CU).  The grid says which: the
-// kernel takes N_CTX / gridDim.x queries per workgroup.  Two wavefronts share each SIMD.  K and
-// V blocks of 64 * 8/QB keys go from global memory straight into an LDS ring (buffer_load ...
-// lds) of 2, 4 or 8 stages, up to seven blocks ahead.
+// Workgroup = QB query blocks of 32 x KG key groups, one wavefront each: 64, 128 or 256
+// queries of one (batch, head) as (QB, KG) = (2,4), (4,2), (8,1) with 512 threads, or 256
+// queries as (8,2) with 1024 threads.  Wavefront w takes query block w % QB and every KG-th
+// 64-key tile, group w / QB; partial (m, l, O) of the key groups are merged through LDS at the
+// end.  Every workgroup walks all keys of its head, so K / V traffic from L2 falls with the
+// queries per workgroup; key groups exist to keep all CUs busy on small problems (the
+// reference's 2 x 2 x 4096 x 64 gives one 64-query workgroup per CU) and, in the 1024-thread
+// form, to put four wavefronts on every SIMD (the tiled path needs 114 registers).  The launch
+// says which: N_CTX / gridDim.x queries per workgroup, blockDim.x threads.  K and V blocks of
+// 64 KG keys go from global memory straight into an LDS ring (buffer_load ... lds) of 2, 4 or
+// 8 stages, up to seven blocks ahead.
 //
 // Arguments: (Q, K, V, Out, sm_scale: f32, ZH: i64, N_CTX: i64)   dims = {ZH, N_CTX}
 //   ZH = batch * heads; N_CTX a multiple of 256; all four tensors [(ZH*N_CTX), 64].
-// Launch: block (512,1,1); grid (N_CTX / q, ZH, 1) with q = 64, 128 or 256.  Other shapes and
-// grids take the one-query-per-lane reference loop of the same kernel (grid-stride, any grid).
+// Launch: grid (N_CTX / q, ZH, 1) with q = 64, 128 or 256 and block (512,1,1), or q = 256 and
+// block (1024,1,1).  Other shapes and launches take the one-query-per-lane reference loop of the
+// same kernel (grid-stride, any grid and block).
 
 #include "device_common.h"
 
@@ -42,8 +45,7 @@ using namespace imexhip;
 
 namespace {
 
-constexpr int kThreads = 512;
-constexpr int kWaves = kThreads / 64;
+constexpr int kMaxThreads = 1024; // 8 or 16 wavefronts per workgroup
 constexpr int D = 64;                 // head dimension
 constexpr int BN = 64;                // keys per tile; a ring stage holds one K and one V tile per key group
 constexpr int kTileBytes = BN * D * 2;          // 8 KiB
@@ -70,20 +72,18 @@ __device__ __forceinline__ float other_half(float v) { return __shfl_xor(v, 32, 
 __device__ __forceinline__ void attention_scalar(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
                                                  uint16_t *Out, float scale, int64_t ZH, int64_t N) {
   const int64_t block = int64_t(blockIdx.z) * gridDim.y * gridDim.x + int64_t(blockIdx.y) * gridDim.x + blockIdx.x;
-  const int64_t stride = int64_t(gridDim.x) * gridDim.y * gridDim.z * kThreads;
+  const int64_t stride = int64_t(gridDim.x) * gridDim.y * gridDim.z * blockDim.x;
   const float c = scale * 1.44269504088896341f;
-  for (int64_t row = block * kThreads + threadIdx.x; row < ZH * N; row += stride) {
+  for (int64_t row = block * blockDim.x + threadIdx.x; row < ZH * N; row += stride) {
     const int64_t head0 = (row / N) * N;
-    float q[D], o[D];
-    for (int d = 0; d < D; ++d) {
-      q[d] = half_bits_to_float(Q[row * D + d]);
+    float o[D]; // the query row is re-read per key (it stays in cache): 64 registers, not 128
+    for (int d = 0; d < D; ++d)
       o[d] = 0.0f;
-    }
     float m = -__builtin_inff(), l = 0.0f;
     for (int64_t j = 0; j < N; ++j) {
       float s = 0.0f;
       for (int d = 0; d < D; ++d)
-        s += q[d] * half_bits_to_float(K[(head0 + j) * D + d]);
+        s += half_bits_to_float(Q[row * D + d]) * half_bits_to_float(K[(head0 + j) * D + d]);
       s *= c;
       const float mNew = fmaxf(m, s);
       const float alpha = exp2f(m - mNew);
@@ -99,21 +99,21 @@ __device__ __forceinline__ void attention_scalar(const uint16_t *Q, const uint16
 }
 
 // ---- MFMA path ---------------------------------------------------------------------------
-// QB = 32-query blocks per workgroup (2, 4 or 8); the 8 wavefronts are QB query blocks x KG = 8 / QB
-// key groups.  More query blocks mean fewer workgroups but proportionally less K / V traffic from L2
-// (every workgroup walks all keys of its head), smaller ring stages and therefore a deeper ring.
-template <int QB>
+// QB = 32-query blocks per workgroup, KG = key groups: QB x KG wavefronts (8 or 16).  More query
+// blocks mean fewer workgroups but proportionally less K / V traffic from L2 (every workgroup walks
+// all keys of its head); fewer key groups mean smaller ring stages and therefore a deeper ring.
+template <int QB, int KG>
 __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K,
                                                 const uint16_t *__restrict__ V, uint16_t *__restrict__ Out,
                                                 float scale, int64_t N, char *lds) {
   LdsChar *ldsBase = (LdsChar *)lds;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  constexpr int KG = kWaves / QB;                  // key groups: wavefronts that split the keys of one query block
+  constexpr int kWaves = QB * KG;
   constexpr int kStageBytes = 2 * KG * kTileBytes; // K tiles of all key groups, then their V tiles
   constexpr int kStages = kLdsBytes / kStageBytes; // 2, 4 or 8
   constexpr int kAhead = kStages - 1;              // blocks in flight ahead of the one being multiplied
-  constexpr int kCopies = KG;                      // 1 KiB copies per wavefront, stage and operand
+  constexpr int kCopies = 64 * KG / (8 * kWaves);  // 1 KiB (8-row) copies per wavefront, stage and operand
   const int wq = wave % QB, wk = wave / QB;
   const int qi = lane & 31, half = lane >> 5;
   // Workgroups go to the 8 XCDs round-robin in launch order, and each XCD has its own L2.  Renumber
@@ -147,8 +147,8 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
   int kVoff[kCopies], vVoff[kCopies];
 #pragma unroll
   for (int c = 0; c < kCopies; ++c) {
-    // wavefront w copies rows [8 KG w, 8 KG (w+1)) of the stage's 64 KG K rows and of its V rows
-    const int row = wave * (8 * KG) + c * 8 + (lane >> 3); // key within the stage's block of 64 KG keys
+    // wavefront w copies rows [8 kCopies w, 8 kCopies (w+1)) of the stage's 64 KG K rows and of its V rows
+    const int row = wave * (8 * kCopies) + c * 8 + (lane >> 3); // key within the stage's block of 64 KG keys
     const int r = row & 63;                          // row within its tile
     const int kc = (lane & 7) ^ ((r ^ ((r >> 3) & 3)) & 7);
     const int vc = (lane & 7) ^ (((r >> 1) & 1) << 2);
@@ -156,7 +156,7 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
     vVoff[c] = (row * D + vc * 8) * 2;
   }
   auto dma_stage = [&](int block, int stage) { // keys [64 KG block, 64 KG (block + 1)) into ring stage `stage`
-    LdsChar *dst = ldsBase + stage * kStageBytes + wave * (KG * 1024);
+    LdsChar *dst = ldsBase + stage * kStageBytes + wave * (kCopies * 1024);
     const int soff = block * (KG * BN * D * 2);
 #pragma unroll
     for (int c = 0; c < kCopies; ++c)
@@ -329,7 +329,7 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
 
 } // namespace
 
-extern "C" __global__ __launch_bounds__(kThreads) void imex_flash_attention_fwd_f16(const uint16_t *Q,
+extern "C" __global__ __launch_bounds__(kMaxThreads) void imex_flash_attention_fwd_f16(const uint16_t *Q,
                                                                                    const uint16_t *K,
                                                                                    const uint16_t *V,
                                                                                    uint16_t *Out, float sm_scale,
@@ -339,12 +339,14 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_flash_attention_fwd_
   const bool shaped = N_CTX > 0 && N_CTX % 256 == 0 && gridDim.y == ZH && gridDim.z == 1 &&
                       ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
                         reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(Out)) & 15) == 0;
-  if (shaped && int64_t(gridDim.x) * 64 == N_CTX)
-    attention_tiled<2>(Q, K, V, Out, sm_scale, N_CTX, lds);
-  else if (shaped && int64_t(gridDim.x) * 128 == N_CTX)
-    attention_tiled<4>(Q, K, V, Out, sm_scale, N_CTX, lds);
-  else if (shaped && int64_t(gridDim.x) * 256 == N_CTX)
-    attention_tiled<8>(Q, K, V, Out, sm_scale, N_CTX, lds);
+  if (shaped && blockDim.x == 512 && int64_t(gridDim.x) * 64 == N_CTX)
+    attention_tiled<2, 4>(Q, K, V, Out, sm_scale, N_CTX, lds);
+  else if (shaped && blockDim.x == 512 && int64_t(gridDim.x) * 128 == N_CTX)
+    attention_tiled<4, 2>(Q, K, V, Out, sm_scale, N_CTX, lds);
+  else if (shaped && blockDim.x == 512 && int64_t(gridDim.x) * 256 == N_CTX)
+    attention_tiled<8, 1>(Q, K, V, Out, sm_scale, N_CTX, lds);
+  else if (shaped && blockDim.x == 1024 && int64_t(gridDim.x) * 256 == N_CTX)
+    attention_tiled<8, 2>(Q, K, V, Out, sm_scale, N_CTX, lds);
   else
     attention_scalar(Q, K, V, Out, sm_scale, ZH, N_CTX);
 }

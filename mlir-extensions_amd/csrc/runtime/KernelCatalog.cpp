@@ -199,9 +199,10 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     break;
   }
   case Shape::Attention: {
-    // dims = {ZH, N_CTX}.  When N_CTX % 256 == 0 a workgroup (8 wavefronts) takes 64, 128 or 256 queries of
-    // one (batch, head); the kernel reads the choice off the grid.  More queries per workgroup mean less
-    // K / V traffic, so: the largest of the three that still gives every one of the 256 CUs a workgroup.
+    // dims = {ZH, N_CTX}.  When N_CTX % 256 == 0 a workgroup takes 64, 128 or 256 queries of one
+    // (batch, head); the kernel reads the choice off the grid and the block.  More queries per workgroup
+    // mean less K / V traffic, so: the largest of the three that still gives every one of the 256 CUs a
+    // workgroup.  256 queries run as sixteen wavefronts (8 query blocks x 2 key groups), the others as eight.
     const int64_t ZH = dims[0], N = dims[1];
     block[0] = 512;
     if (N > 0 && N % 256 == 0 && ZH > 0 && ZH <= 65535) {
@@ -210,6 +211,8 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
         queries /= 2;
       grid[0] = static_cast<size_t>(N / queries);
       grid[1] = static_cast<size_t>(ZH);
+      if (queries == 256)
+        block[0] = 1024;
     } else {
       grid[0] = ceilDiv(ZH * N, 512); // one lane per query
     }

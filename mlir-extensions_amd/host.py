@@ -225,11 +225,12 @@ class Stream:
         module = self.rt.gpuModuleLoad(self.handle, blob, size.value)
         return self.rt.gpuKernelGet(self.handle, module, name.encode())
 
-    def launch(self, name, dims, args, deps=None, grid=None):
+    def launch(self, name, dims, args, deps=None, grid=None, block=None):
         """gpuModuleLoad + gpuKernelGet + gpuLaunchKernel; returns the event (or
-        None when the launch shape is empty).  `grid` replaces the catalogue's grid."""
-        cat_grid, block, smem = launch_shape(name, dims)
+        None when the launch shape is empty).  `grid` / `block` replace the catalogue's."""
+        cat_grid, cat_block, smem = launch_shape(name, dims)
         grid = tuple(grid) if grid is not None else cat_grid
+        block = tuple(block) if block is not None else cat_block
         if 0 in grid:
             return None
         fn = self.kernel(name)
@@ -368,10 +369,11 @@ def input_fusion(stream, a, b, dtype="f32"):
     return _binary(stream, "imex_input_fusion_" + dtype, a, b, dtype, [rows, cols], (cols,))
 
 
-def flash_attention(stream, q, k, v, zh, n_ctx, sm_scale, queries_per_workgroup=None):
+def flash_attention(stream, q, k, v, zh, n_ctx, sm_scale, queries_per_workgroup=None, threads=512):
     """WG/flash_attention_fwd.mlir:25-307: softmax(sm_scale * Q K^T) V per (batch, head);
     q, k, v f16 bit patterns [(zh * n_ctx), 64].  `queries_per_workgroup` (64, 128 or 256,
-    n_ctx a multiple of 256) picks the tiling instead of the catalogue."""
+    n_ctx a multiple of 256) picks the tiling instead of the catalogue; 256 queries also come
+    with `threads` = 1024 (sixteen wavefronts, two key groups)."""
     for t in (q, k, v):
         _check(t, "f16")
         if t.shape != (zh * n_ctx, 64):
@@ -379,13 +381,15 @@ def flash_attention(stream, q, k, v, zh, n_ctx, sm_scale, queries_per_workgroup=
     d_q, d_k, d_v = stream.to_device(q), stream.to_device(k), stream.to_device(v)
     d_o = stream.alloc(max(q.size, 1) * 2)
     try:
-        grid = None
+        grid = block = None
         if queries_per_workgroup is not None:
             if queries_per_workgroup not in (64, 128, 256) or n_ctx % 256:
                 raise ValueError("queries_per_workgroup must be 64, 128 or 256 and n_ctx a multiple of 256")
-            grid = (n_ctx // queries_per_workgroup, zh, 1)
+            if threads not in (512, 1024) or (threads == 1024 and queries_per_workgroup != 256):
+                raise ValueError("threads is 512, or 1024 with 256 queries per workgroup")
+            grid, block = (n_ctx // queries_per_workgroup, zh, 1), (threads, 1, 1)
         stream.launch("imex_flash_attention_fwd_f16", [zh, n_ctx], [d_q, d_k, d_v, d_o, float(sm_scale), zh, n_ctx],
-                      grid=grid)
+                      grid=grid, block=block)
         stream.wait()
         return stream.from_device(d_o, q.shape, np.uint16)
     finally:

@@ -378,17 +378,18 @@ def test_flash_attention_sixteen_heads(host, orc, stream):
 @pytest.mark.parametrize("zh,n_ctx,scale", [(3, 512, 0.5), (2, 256, 4.0), (1, 2048, 0.125)])
 def test_flash_attention_every_tiling(host, orc, stream, zh, n_ctx, scale):
     """64, 128 and 256 queries per workgroup (2, 4, 8 query blocks x 4, 2, 1 key groups; ring of
-    2, 4, 8 stages): each against the oracle, on the same inputs."""
+    2, 4, 8 stages) and 256 queries as sixteen wavefronts (8 x 2, ring of 4): each against the
+    oracle, on the same inputs."""
     n = zh * n_ctx
     q = orc.fill_uniform(n * 64, "f16", 71, -2, 2).reshape(n, 64)
     k = orc.fill_uniform(n * 64, "f16", 72, -2, 2).reshape(n, 64)
     v = orc.fill_uniform(n * 64, "f16", 73, -1, 1).reshape(n, 64)
     rows = np.unique(np.concatenate([np.arange(0, n, 7), [n_ctx - 1, n - 1]]))
     ref = orc.flash_attention_rows(q, k, v, n_ctx, scale, rows)
-    for queries in (64, 128, 256):
-        say("attention %dx%d, %d queries per workgroup" % (zh, n_ctx, queries))
-        got = host.flash_attention(stream, q, k, v, zh, n_ctx, scale, queries_per_workgroup=queries)
-        assert attention_close(got[rows], ref, orc), queries
+    for queries, threads in ((64, 512), (128, 512), (256, 512), (256, 1024)):
+        say("attention %dx%d, %d queries per workgroup of %d threads" % (zh, n_ctx, queries, threads))
+        got = host.flash_attention(stream, q, k, v, zh, n_ctx, scale, queries_per_workgroup=queries, threads=threads)
+        assert attention_close(got[rows], ref, orc), (queries, threads)
 
 
 @pytest.mark.parametrize("zh", [8, 16])
@@ -396,7 +397,8 @@ def test_flash_attention_catalogue_picks_wide_tilings(host, orc, stream, zh):
     """N_CTX = 4096 with 8 and 16 heads: the catalogue launches 128- and 256-query workgroups
     (16 heads is the reference's flash_attention_fwd_ov_with_arrray_len_4k.mlir shape)."""
     n_ctx = 4096
-    assert host.launch_shape("imex_flash_attention_fwd_f16", [zh, n_ctx])[0] == (n_ctx // (16 * zh), zh, 1)
+    grid, block, _ = host.launch_shape("imex_flash_attention_fwd_f16", [zh, n_ctx])
+    assert grid == (n_ctx // (16 * zh), zh, 1) and block == ((1024 if zh == 16 else 512), 1, 1)
     n = zh * n_ctx
     q = orc.fill_uniform(n * 64, "f16", 74, -1, 1).reshape(n, 64)
     k = orc.fill_uniform(n * 64, "f16", 75, -1, 1).reshape(n, 64)

@@ -95,8 +95,8 @@ def test_launch_shapes(host):
     assert ls("imex_flash_attention_fwd_f16", [2, 100])[0] == (1, 1, 1)
     # 64, 128 or 256 queries per workgroup: the most that still leaves 256 workgroups
     assert ls("imex_flash_attention_fwd_f16", [8, 4096])[0] == (32, 8, 1)
-    assert ls("imex_flash_attention_fwd_f16", [16, 4096])[0] == (16, 16, 1)
-    assert ls("imex_flash_attention_fwd_f16", [64, 1024])[0] == (4, 64, 1)
+    assert ls("imex_flash_attention_fwd_f16", [16, 4096])[:2] == ((16, 16, 1), (1024, 1, 1))  # 256 queries: 16 wavefronts
+    assert ls("imex_flash_attention_fwd_f16", [64, 1024])[:2] == ((4, 64, 1), (1024, 1, 1))
     assert ls("imex_flash_attention_fwd_f16", [3, 256])[0] == (4, 3, 1)
     assert ls("imex_input_fusion_f32", [512, 1024])[0] == (4, 1, 1)
     assert ls("imex_gemm_4kx4kx4k_transpose_a", []) == ((16, 16, 1), (512, 1, 1), 0)
