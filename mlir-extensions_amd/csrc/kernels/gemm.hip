@@ -381,7 +381,13 @@ __device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B,
   // The MFMA path wants K in whole 32-wide steps and 16-byte aligned rows in memory: a row of
   // B [K,N] (or of A [K,M] when transposed) is N (M) elements long, so those must be multiples
   // of 8.  M and N need not divide the tile: edge tiles multiply padding and store what exists.
+  // An operand whose rows are strided in memory is addressed with 32-bit byte offsets from one
+  // buffer descriptor, so it has to stay below 2 GiB; a k-contiguous one below 4 Mi elements per row.
+  constexpr int64_t kMaxBytes = int64_t(1) << 31, kMaxRow = int64_t(1) << 22;
+  const bool fitsA = kAT ? K * M * 2 < kMaxBytes : K < kMaxRow;
+  const bool fitsB = kBT ? K < kMaxRow : K * N * 2 < kMaxBytes;
   const bool tileable = M > 0 && N > 0 && K > 0 && K % RK == 0 && (kBT || N % 8 == 0) && (!kAT || M % 8 == 0) &&
+                        fitsA && fitsB &&
                         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
   if (tileable)
     gemm_tiled<T, kAT, kBT, Epi>(A, B, M, N, K, epi, lds);

@@ -230,7 +230,11 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     const int64_t M = dims[0], N = dims[1], K = dims[2];
     const bool rowsB = e->shape == Shape::GemmTB || N % 8 == 0;
     const bool rowsA = e->shape != Shape::GemmTA || M % 8 == 0;
-    const bool tileable = M > 0 && N > 0 && K > 0 && K % 32 == 0 && rowsA && rowsB;
+    // operands addressed through one 32-bit-offset buffer descriptor must stay below 2 GiB
+    const int64_t twoGiB = int64_t(1) << 31, maxRow = int64_t(1) << 22;
+    const bool fitsA = e->shape == Shape::GemmTA ? K * M * 2 < twoGiB : K < maxRow;
+    const bool fitsB = e->shape == Shape::GemmTB ? K < maxRow : K * N * 2 < twoGiB;
+    const bool tileable = M > 0 && N > 0 && K > 0 && K % 32 == 0 && rowsA && rowsB && fitsA && fitsB;
     block[0] = 512;
     grid[0] = tileable ? ceilDiv(M, 256) * ceilDiv(N, 256) : ceilDiv(M * N, 512);
     break;

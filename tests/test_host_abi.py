@@ -90,6 +90,10 @@ def test_launch_shapes(host):
     assert ls("imex_gemm_f16_f16_f32_tb", [256, 252, 64])[0] == (1, 1, 1)  # B stored [N,K]: any N
     assert ls("imex_gemm_f16_f16_f32_ta", [252, 256, 64])[0] == (126, 1, 1)  # A stored [K,M]: M % 8 != 0
     assert ls("imex_gemm_f16_f16_f32_ta", [248, 256, 64])[0] == (1, 1, 1)
+    # a strided operand of 2 GiB or more cannot be addressed with 32-bit offsets: one lane per output
+    assert ls("imex_gemm_f16_f16_f32", [256, 32768, 32768])[0] == (256 * 32768 // 512, 1, 1)
+    assert ls("imex_gemm_f16_f16_f32", [256, 32768, 32736])[0] == (128, 1, 1)
+    assert ls("imex_gemm_f16_f16_f32_tb", [256, 32768, 32768])[0] == (128, 1, 1)
     assert ls("imex_gemm_4kx4kx4k_f16_f16_f32", []) == ((16, 16, 1), (512, 1, 1), 0)
     assert ls("imex_flash_attention_fwd_f16", [4, 4096]) == ((64, 4, 1), (512, 1, 1), 0)
     assert ls("imex_flash_attention_fwd_f16", [2, 100])[0] == (1, 1, 1)
