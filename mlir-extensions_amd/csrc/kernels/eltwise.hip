@@ -28,21 +28,23 @@ __device__ __forceinline__ void stream_map_impl(const void *__restrict__ in, voi
                                                 Op op) {
   constexpr int kElemsPerVec = 16 / kElemBytes;
   constexpr int64_t kElemsPerBlock = int64_t(kThreads) * kVecsPerThread * kElemsPerVec;
-  const int64_t base = int64_t(blockIdx.x) * kElemsPerBlock;
   const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-  if (aligned && base + kElemsPerBlock <= n) {
-    const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(in) + base * kElemBytes);
-    u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + base * kElemBytes);
-    u32x4 v[kVecsPerThread];
+  // workgroups stride over the blocks, so a grid smaller than ceil(n / kElemsPerBlock) still covers n
+  for (int64_t base = int64_t(blockIdx.x) * kElemsPerBlock; base < n; base += int64_t(gridDim.x) * kElemsPerBlock) {
+    if (aligned && base + kElemsPerBlock <= n) {
+      const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(in) + base * kElemBytes);
+      u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + base * kElemBytes);
+      u32x4 v[kVecsPerThread];
 #pragma unroll
-    for (int j = 0; j < kVecsPerThread; ++j)
-      v[j] = load128<kStream>(src + j * kThreads + threadIdx.x);
+      for (int j = 0; j < kVecsPerThread; ++j)
+        v[j] = load128<kStream>(src + j * kThreads + threadIdx.x);
 #pragma unroll
-    for (int j = 0; j < kVecsPerThread; ++j)
-      store128<kStream>(op.vec(v[j]), dst + j * kThreads + threadIdx.x);
-  } else {
-    for (int64_t i = base + threadIdx.x; i < base + kElemsPerBlock && i < n; i += kThreads)
-      op.scalar(in, out, i);
+      for (int j = 0; j < kVecsPerThread; ++j)
+        store128<kStream>(op.vec(v[j]), dst + j * kThreads + threadIdx.x);
+    } else {
+      for (int64_t i = base + threadIdx.x; i < base + kElemsPerBlock && i < n; i += kThreads)
+        op.scalar(in, out, i);
+    }
   }
 }
 

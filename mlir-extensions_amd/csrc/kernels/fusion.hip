@@ -61,8 +61,10 @@ __device__ __forceinline__ float logf_libm(float x, const LogfEntry *table) {
       return -__builtin_inff(); // log(+-0)
     if (ix == 0x7f800000u)
       return x;                 // log(inf)
-    if ((ix & 0x80000000u) || ix * 2 >= 0xff000000u)
-      return __builtin_nanf(""); // negative or NaN
+    if (ix * 2 > 0xff000000u)
+      return x + x;             // NaN: quieted, sign and payload kept
+    if (ix & 0x80000000u)
+      return u2f(0xffc00000u);  // log of a negative number: libm's (x - x) / 0, the x86 default NaN
     ix = f2u(x * 0x1p23f);      // subnormal: normalise
     ix -= 23u << 23;
   }
@@ -146,32 +148,34 @@ __device__ __forceinline__ void loop_fusion(const void *__restrict__ a, const vo
   __shared__ LogfEntry table[16];
   stage_table(table);
   constexpr int64_t kElemsPerBlock = int64_t(kThreads) * kVecsPerThread * E::kPerVec;
-  const int64_t base = int64_t(blockIdx.x) * kElemsPerBlock;
   const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
                          reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-  if (aligned && base + kElemsPerBlock <= n) {
-    const u32x4 *pa = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a) + base * E::kBytes);
-    const u32x4 *pb = reinterpret_cast<const u32x4 *>(static_cast<const char *>(b) + base * E::kBytes);
-    u32x4 *po = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + base * E::kBytes);
-    u32x4 va[kVecsPerThread], vb[kVecsPerThread];
+  // workgroups stride over the blocks, so any grid covers n
+  for (int64_t base = int64_t(blockIdx.x) * kElemsPerBlock; base < n; base += int64_t(gridDim.x) * kElemsPerBlock) {
+    if (aligned && base + kElemsPerBlock <= n) {
+      const u32x4 *pa = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a) + base * E::kBytes);
+      const u32x4 *pb = reinterpret_cast<const u32x4 *>(static_cast<const char *>(b) + base * E::kBytes);
+      u32x4 *po = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + base * E::kBytes);
+      u32x4 va[kVecsPerThread], vb[kVecsPerThread];
 #pragma unroll
-    for (int j = 0; j < kVecsPerThread; ++j) {
-      va[j] = load128<true>(pa + j * kThreads + threadIdx.x);
-      vb[j] = load128<true>(pb + j * kThreads + threadIdx.x);
+      for (int j = 0; j < kVecsPerThread; ++j) {
+        va[j] = load128<true>(pa + j * kThreads + threadIdx.x);
+        vb[j] = load128<true>(pb + j * kThreads + threadIdx.x);
+      }
+#pragma unroll
+      for (int j = 0; j < kVecsPerThread; ++j) {
+        float fa[E::kPerVec], fb[E::kPerVec];
+        E::unpack(va[j], fa);
+        E::unpack(vb[j], fb);
+#pragma unroll
+        for (int i = 0; i < E::kPerVec; ++i)
+          fa[i] = loop_chain(fa[i], fb[i], table);
+        store128<true>(E::pack(fa), po + j * kThreads + threadIdx.x);
+      }
+    } else {
+      for (int64_t i = base + threadIdx.x; i < base + kElemsPerBlock && i < n; i += kThreads)
+        E::put(out, i, loop_chain(E::get(a, i), E::get(b, i), table));
     }
-#pragma unroll
-    for (int j = 0; j < kVecsPerThread; ++j) {
-      float fa[E::kPerVec], fb[E::kPerVec];
-      E::unpack(va[j], fa);
-      E::unpack(vb[j], fb);
-#pragma unroll
-      for (int i = 0; i < E::kPerVec; ++i)
-        fa[i] = loop_chain(fa[i], fb[i], table);
-      store128<true>(E::pack(fa), po + j * kThreads + threadIdx.x);
-    }
-  } else {
-    for (int64_t i = base + threadIdx.x; i < base + kElemsPerBlock && i < n; i += kThreads)
-      E::put(out, i, loop_chain(E::get(a, i), E::get(b, i), table));
   }
 }
 

@@ -77,28 +77,29 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_rowsum_f32(const flo
   const int wave = threadIdx.x / kWave;
   // the input is read exactly once: stream it past the caches (non-temporal)
   constexpr bool stream = true;
+  // workgroups (wavefronts) stride over the rows, so any grid covers all of them
   if (cols > kWavePerRowMaxCols) {
     __shared__ float partial[kWavesPerBlock];
-    const int64_t row = blockIdx.x;
-    if (row >= rows)
-      return;
-    const float p = stream ? row_partial<true>(in + row * cols, cols, threadIdx.x, kThreads)
-                           : row_partial<false>(in + row * cols, cols, threadIdx.x, kThreads);
-    float s = wave_sum(p);
-    if (lane == 0)
-      partial[wave] = s;
-    __syncthreads();
-    if (threadIdx.x == 0)
-      out[row] = init + ((partial[0] + partial[1]) + (partial[2] + partial[3]));
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+      const float p = stream ? row_partial<true>(in + row * cols, cols, threadIdx.x, kThreads)
+                             : row_partial<false>(in + row * cols, cols, threadIdx.x, kThreads);
+      float s = wave_sum(p);
+      if (lane == 0)
+        partial[wave] = s;
+      __syncthreads();
+      if (threadIdx.x == 0)
+        out[row] = init + ((partial[0] + partial[1]) + (partial[2] + partial[3]));
+      __syncthreads(); // `partial` is reused by the next row
+    }
   } else {
-    const int64_t row = int64_t(blockIdx.x) * kWavesPerBlock + wave;
-    if (row >= rows)
-      return;
-    const float p = stream ? row_partial<true>(in + row * cols, cols, lane, kWave)
-                           : row_partial<false>(in + row * cols, cols, lane, kWave);
-    float s = wave_sum(p);
-    if (lane == 0)
-      out[row] = init + s;
+    for (int64_t row = int64_t(blockIdx.x) * kWavesPerBlock + wave; row < rows;
+         row += int64_t(gridDim.x) * kWavesPerBlock) {
+      const float p = stream ? row_partial<true>(in + row * cols, cols, lane, kWave)
+                             : row_partial<false>(in + row * cols, cols, lane, kWave);
+      float s = wave_sum(p);
+      if (lane == 0)
+        out[row] = init + s;
+    }
   }
 }
 

@@ -202,6 +202,37 @@ def test_reduce_outer_benchmark_shape_and_any_grid(host, orc, stream):
     assert np.array_equal(out, 1.0 + small.sum(axis=0, dtype=np.float64).astype(np.float32))
 
 
+@pytest.mark.parametrize("grid", [(3, 1, 1), (100000, 1, 1)])
+def test_streaming_kernels_any_grid(host, orc, stream, grid):
+    """relu, silu, softmax, row sum and the fused chain stride over their work: a grid much
+    smaller or much larger than the catalogue's gives the same bits."""
+    n = 3 * 4096 * 5 + 77
+    x = orc.fill_uniform(n, "f32", 91, -3, 3)
+    for kernel, ref in (("imex_relu_f32", orc.relu_f32(x)), ("imex_silu_f32", orc.silu_f32(x))):
+        d_in, d_out = stream.to_device(x), stream.alloc(n * 4)
+        stream.launch(kernel, [n], [d_in, d_out, n], grid=grid)
+        stream.wait()
+        got = stream.from_device(d_out, (n,), np.float32)
+        stream.free(d_in), stream.free(d_out)
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), kernel
+    for rows, cols in ((37, 3000), (1000, 300)):
+        m = orc.fill_int(rows * cols, "f32", 92, -8, 8).reshape(rows, cols)
+        d_in, d_out = stream.to_device(m), stream.alloc(rows * 4)
+        stream.launch("imex_rowsum_f32", [rows, cols], [d_in, d_out, rows, cols, 2.0], grid=grid)
+        stream.wait()
+        got = stream.from_device(d_out, (rows,), np.float32)
+        stream.free(d_in), stream.free(d_out)
+        assert np.array_equal(got, 2.0 + m.sum(axis=1, dtype=np.float64).astype(np.float32)), (rows, cols)
+    a = np.abs(orc.fill_uniform(n, "f32", 93, -3, 3)) + 0.5
+    d_a, d_b, d_out = stream.to_device(x), stream.to_device(a), stream.alloc(n * 4)
+    stream.launch("imex_loop_fusion_f32", [n], [d_a, d_b, d_out, n], grid=grid)
+    stream.wait()
+    got = stream.from_device(d_out, (n,), np.float32)
+    for p in (d_a, d_b, d_out):
+        stream.free(p)
+    assert np.array_equal(got.view(np.uint32), orc.loop_fusion_f32(x, a).view(np.uint32))
+
+
 # =============================== Transpose =================================
 def test_transpose_golden(host, orc, stream):
     g = GOLD["transpose_f32_10x20"]
