@@ -42,7 +42,7 @@
 // reference's CPU loop (lib/ExecutionEngine/ImexRunnerUtils.cpp:308-317).
 //
 // Launch: block (512,1,1); grid (tiles,1,1) with tiles = ceil(M/256)*ceil(N/256) on
-// the MFMA path, else (ceil(M*N/512),1,1).  The fixed-shape 4096^3 entry
+// the MFMA path, else (ceil(M*N/512),1,1); workgroups stride, so any grid is correct.  The fixed-shape 4096^3 entry
 // points take the reference's own launch: blocks (16,16,1), threads (512,1,1).
 
 #include "device_common.h"
@@ -262,9 +262,11 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
   // -- workgroup id -> tile, XCD-aware ------------------------------------------------
   const int tilesM = int((M + BM - 1) / BM), tilesN = int((N + BN - 1) / BN);
   const int tiles = tilesM * tilesN;
-  int pid = blockIdx.y * gridDim.x + blockIdx.x;
-  if (pid >= tiles)
-    return; // a launch with more workgroups than tiles: the surplus has nothing to do
+  // Workgroups stride over the tiles: a launch with fewer workgroups than tiles still covers C, one
+  // with more leaves the surplus nothing to do.
+  const int workgroups = gridDim.x * gridDim.y;
+  for (int id = blockIdx.y * gridDim.x + blockIdx.x; id < tiles; id += workgroups) {
+  int pid = id;
   if (tiles % 8 == 0)
     pid = (pid % 8) * (tiles / 8) + pid / 8; // ids congruent mod 8 share an XCD
   const int group = kGroupM * tilesN;
@@ -371,6 +373,9 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
             epi(m, n, N, acc[i][j][r]);
         }
   }
+  if (id + workgroups < tiles)
+    __syncthreads(); // the ring is reused by this workgroup's next tile
+  } // tiles of this workgroup
 }
 
 template <typename T, bool kAT, bool kBT, typename Epi>

@@ -599,10 +599,11 @@ def test_gemm_ragged_tiles_transposed_operands(host, orc, stream, which, M, N, K
 
 
 def test_gemm_launch_shape_slack(host, orc, stream):
-    """A grid with more workgroups than tiles (tiled path) or fewer threads than
-    outputs (one-thread-per-output path) still computes every element once."""
+    """A grid with more or fewer workgroups than tiles (MFMA path: the workgroups stride
+    over the tiles) or fewer threads than outputs (one-thread-per-output path) still
+    computes every element once."""
     import ctypes as C
-    for (M, N, K, grid) in [(256, 256, 64, 9), (100, 36, 130, 2)]:
+    for (M, N, K, grid) in [(256, 256, 64, 9), (100, 36, 130, 2), (1024, 768, 96, 5), (1000, 520, 64, 1)]:
         a = orc.fill_uniform(M * K, "f16", 21, -1, 1).reshape(M, K)
         b = orc.fill_uniform(K * N, "f16", 22, -1, 1).reshape(K, N)
         d_a, d_b, d_c = stream.to_device(a), stream.to_device(b), stream.alloc(M * N * 4)
