@@ -34,10 +34,11 @@
 // 8 stages, up to seven blocks ahead.
 //
 // Arguments: (Q, K, V, Out, sm_scale: f32, ZH: i64, N_CTX: i64)   dims = {ZH, N_CTX}
-//   ZH = batch * heads; N_CTX a multiple of 256; all four tensors [(ZH*N_CTX), 64].
-// Launch: grid (N_CTX / q, ZH, 1) with q = 64, 128 or 256 and block (512,1,1), or q = 256 and
-// block (1024,1,1).  Other shapes and launches take the one-query-per-lane reference loop of the
-// same kernel (grid-stride, any grid and block).
+//   ZH = batch * heads; all four tensors [(ZH*N_CTX), 64]; sm_scale > 0.  N_CTX need not divide the
+//   tiles: queries past the end are not stored, keys past the end get a score of -inf.
+// Launch: grid (ceil(N_CTX / q), ZH, 1) with q = 64, 128 or 256 and block (512,1,1), or q = 256
+// and block (1024,1,1).  Other launches (and a scale <= 0, or misaligned tensors) take the
+// one-query-per-lane reference loop of the same kernel (grid-stride, any grid and block).
 
 #include "device_common.h"
 
@@ -102,7 +103,9 @@ __device__ __forceinline__ void attention_scalar(const uint16_t *Q, const uint16
 // QB = 32-query blocks per workgroup, KG = key groups: QB x KG wavefronts (8 or 16).  More query
 // blocks mean fewer workgroups but proportionally less K / V traffic from L2 (every workgroup walks
 // all keys of its head); fewer key groups mean smaller ring stages and therefore a deeper ring.
-template <int QB, int KG>
+// kRagged: N_CTX is not a multiple of the workgroup's 32 QB queries or of its 64 KG-key blocks; the
+// padding logic below is compiled in only then.
+template <int QB, int KG, bool kRagged>
 __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K,
                                                 const uint16_t *__restrict__ V, uint16_t *__restrict__ Out,
                                                 float scale, int64_t N, char *lds) {
@@ -130,12 +133,16 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
   }
   const int64_t head0 = int64_t(by) * N;                 // first row of this (batch, head)
   const int64_t q0 = head0 + int64_t(bx) * (32 * QB) + wq * 32;
+  // N_CTX need not divide the tiles.  Queries past the end of the head are computed on a copy of
+  // its last row and not stored; keys past the end are copies of the last key whose scores are
+  // set to -inf before the softmax (below), so no address ever leaves the head.
+  const int64_t qRow = kRagged ? min(q0 + qi, head0 + N - 1) : q0 + qi;
 
   // Q^T operand: lane (q, half) keeps Q[q][ds*16 + half*8 .. +7] for the four 16-wide steps
   f16x8 qf[4];
 #pragma unroll
   for (int ds = 0; ds < 4; ++ds)
-    qf[ds] = *reinterpret_cast<const f16x8 *>(Q + (q0 + qi) * D + ds * 16 + half * 8);
+    qf[ds] = *reinterpret_cast<const f16x8 *>(Q + qRow * D + ds * 16 + half * 8);
 
   // -- global -> LDS copies.  A stage is [K tile 0 .. KG-1][V tile 0 .. KG-1], each 64
   // rows of 128 bytes; one copy = 8 rows.  16-byte chunk c of row r is stored at
@@ -144,7 +151,11 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
   // applied on the global side, since a direct copy fixes the lane's LDS position.
   const __amdgpu_buffer_rsrc_t kRsrc = make_rsrc(K + head0 * D, N * D * 2);
   const __amdgpu_buffer_rsrc_t vRsrc = make_rsrc(V + head0 * D, N * D * 2);
-  int kVoff[kCopies], vVoff[kCopies];
+  const int iters = int((N + KG * BN - 1) / (KG * BN));            // key blocks of 64 KG keys
+  const int lastRows = int(N - int64_t(iters - 1) * (KG * BN));    // keys in the last block: 1 .. 64 KG
+  const bool raggedKeys = kRagged && lastRows != KG * BN;
+  int kVoff[kCopies], vVoff[kCopies];   // per-lane byte offsets inside a block
+  int kVoffT[kCopies], vVoffT[kCopies]; // the same for the last block, rows clamped to its last key
 #pragma unroll
   for (int c = 0; c < kCopies; ++c) {
     // wavefront w copies rows [8 kCopies w, 8 kCopies (w+1)) of the stage's 64 KG K rows and of its V rows
@@ -154,16 +165,21 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
     const int vc = (lane & 7) ^ (((r >> 1) & 1) << 2);
     kVoff[c] = (row * D + kc * 8) * 2;
     vVoff[c] = (row * D + vc * 8) * 2;
+    const int rowT = kRagged ? min(row, lastRows - 1) : row;
+    kVoffT[c] = (rowT * D + kc * 8) * 2;
+    vVoffT[c] = (rowT * D + vc * 8) * 2;
   }
   auto dma_stage = [&](int block, int stage) { // keys [64 KG block, 64 KG (block + 1)) into ring stage `stage`
     LdsChar *dst = ldsBase + stage * kStageBytes + wave * (kCopies * 1024);
     const int soff = block * (KG * BN * D * 2);
+    const bool tail = raggedKeys && block == iters - 1; // uniform
 #pragma unroll
     for (int c = 0; c < kCopies; ++c)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(kRsrc, dst + c * 1024, 16, kVoff[c], soff, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kRsrc, dst + c * 1024, 16, tail ? kVoffT[c] : kVoff[c], soff, 0, 0);
 #pragma unroll
     for (int c = 0; c < kCopies; ++c)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(vRsrc, dst + KG * kTileBytes + c * 1024, 16, vVoff[c], soff, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vRsrc, dst + KG * kTileBytes + c * 1024, 16,
+                                               tail ? vVoffT[c] : vVoff[c], soff, 0, 0);
   };
 
   // -- LDS read addresses (relative to this wavefront's K / V tile of a stage)
@@ -201,7 +217,6 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
 
   // The ring always holds kAhead blocks in flight (past the end the last block is simply fetched
   // again, into stages nobody reads any more), so "block `it` has landed" is one fixed vmcnt.
-  const int iters = int(N / (KG * BN));
 #pragma unroll
   for (int b = 0; b < kAhead; ++b)
     dma_stage(min(b, iters - 1), b);
@@ -231,6 +246,15 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
         for (int kb = 0; kb < 2; ++kb)
           s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[kb][ds], qf[ds], ds == 0 ? zero : s[kb], 0, 0, 0);
     }
+    // keys of this wavefront's tile that exist: fewer than 64 only in the last block of a ragged N_CTX
+    const int nValid = int(N) - (it * (KG * BN) + wk * BN);
+    if (kRagged && nValid < BN) { // uniform over the wavefront
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          s[kb][r] = kb * 32 + (r >> 2) * 8 + half * 4 + (r & 3) < nValid ? s[kb][r] : -__builtin_inff();
+    }
     // online softmax over the keys; this lane owns 32 of the query's 64 scores
     float mx = s[0][0];
 #pragma unroll
@@ -239,9 +263,12 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
       for (int r = 0; r < 16; ++r)
         mx = fmaxf(mx, s[kb][r]);
     mx = fmaxf(mx, other_half(mx));
-    const float mNew = fmaxf(m, mx * c);
+    const float mRun = fmaxf(m, mx * c);
+    // a key group that has seen no key yet (ragged N_CTX shorter than its first tile) stays at -inf;
+    // 0 stands in for it below so that -inf - -inf never forms: every p and alpha is then exp2(-inf) = 0
+    const float mNew = kRagged && mRun == -__builtin_inff() ? 0.0f : mRun;
     const float alpha = __builtin_amdgcn_exp2f(m - mNew);
-    m = mNew;
+    m = mRun;
     float sum = 0.0f;
     f16x8 pf[4];
 #pragma unroll
@@ -322,7 +349,8 @@ __device__ __forceinline__ void attention_tiled(const uint16_t *__restrict__ Q, 
             acc += xchg[g * kSlot + (db * 16 + r) * 64 + lane] * a[g + 1];
           out4[e] = static_cast<_Float16>(acc * inv);
         }
-        *reinterpret_cast<f16x4 *>(Out + (q0 + qi) * D + db * 32 + g4 * 8 + half * 4) = out4;
+        if (!kRagged || q0 + qi < head0 + N)
+          *reinterpret_cast<f16x4 *>(Out + (q0 + qi) * D + db * 32 + g4 * 8 + half * 4) = out4;
       }
   }
 }
@@ -335,18 +363,35 @@ extern "C" __global__ __launch_bounds__(kMaxThreads) void imex_flash_attention_f
                                                                                    uint16_t *Out, float sm_scale,
                                                                                    int64_t ZH, int64_t N_CTX) {
   __shared__ __attribute__((aligned(16))) char lds[kLdsBytes];
-  // The grid says how many queries a workgroup takes: N_CTX / gridDim.x = 64, 128 or 256.
-  const bool shaped = N_CTX > 0 && N_CTX % 256 == 0 && gridDim.y == ZH && gridDim.z == 1 &&
+  // The launch says how many queries a workgroup takes (ceil(N_CTX / gridDim.x) = 64, 128 or 256) and
+  // with how many wavefronts.  The tiled path assumes a positive scale (it takes the row maximum
+  // before scaling) and 32-bit byte offsets inside one head.
+  const bool shaped = N_CTX > 0 && N_CTX < (int64_t(1) << 24) && sm_scale > 0.0f && gridDim.y == ZH && gridDim.z == 1 &&
                       ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
                         reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(Out)) & 15) == 0;
-  if (shaped && blockDim.x == 512 && int64_t(gridDim.x) * 64 == N_CTX)
-    attention_tiled<2, 4>(Q, K, V, Out, sm_scale, N_CTX, lds);
-  else if (shaped && blockDim.x == 512 && int64_t(gridDim.x) * 128 == N_CTX)
-    attention_tiled<4, 2>(Q, K, V, Out, sm_scale, N_CTX, lds);
-  else if (shaped && blockDim.x == 512 && int64_t(gridDim.x) * 256 == N_CTX)
-    attention_tiled<8, 1>(Q, K, V, Out, sm_scale, N_CTX, lds);
-  else if (shaped && blockDim.x == 1024 && int64_t(gridDim.x) * 256 == N_CTX)
-    attention_tiled<8, 2>(Q, K, V, Out, sm_scale, N_CTX, lds);
-  else
+  const int64_t gx = gridDim.x;
+  const bool even = N_CTX % 256 == 0; // every tiling divides it
+  if (shaped && blockDim.x == 512 && gx == (N_CTX + 63) / 64) {
+    if (even)
+      attention_tiled<2, 4, false>(Q, K, V, Out, sm_scale, N_CTX, lds);
+    else
+      attention_tiled<2, 4, true>(Q, K, V, Out, sm_scale, N_CTX, lds);
+  } else if (shaped && blockDim.x == 512 && gx == (N_CTX + 127) / 128) {
+    if (even)
+      attention_tiled<4, 2, false>(Q, K, V, Out, sm_scale, N_CTX, lds);
+    else
+      attention_tiled<4, 2, true>(Q, K, V, Out, sm_scale, N_CTX, lds);
+  } else if (shaped && blockDim.x == 512 && gx == (N_CTX + 255) / 256) {
+    if (even)
+      attention_tiled<8, 1, false>(Q, K, V, Out, sm_scale, N_CTX, lds);
+    else
+      attention_tiled<8, 1, true>(Q, K, V, Out, sm_scale, N_CTX, lds);
+  } else if (shaped && blockDim.x == 1024 && gx == (N_CTX + 255) / 256) {
+    if (even)
+      attention_tiled<8, 2, false>(Q, K, V, Out, sm_scale, N_CTX, lds);
+    else
+      attention_tiled<8, 2, true>(Q, K, V, Out, sm_scale, N_CTX, lds);
+  } else {
     attention_scalar(Q, K, V, Out, sm_scale, ZH, N_CTX);
+  }
 }

@@ -199,17 +199,17 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     break;
   }
   case Shape::Attention: {
-    // dims = {ZH, N_CTX}.  When N_CTX % 256 == 0 a workgroup takes 64, 128 or 256 queries of one
-    // (batch, head); the kernel reads the choice off the grid and the block.  More queries per workgroup
-    // mean less K / V traffic, so: the largest of the three that still gives every one of the 256 CUs a
-    // workgroup.  256 queries run as sixteen wavefronts (8 query blocks x 2 key groups), the others as eight.
+    // dims = {ZH, N_CTX}.  A workgroup takes 64, 128 or 256 queries of one (batch, head); the kernel reads
+    // the choice off the grid and the block.  More queries per workgroup mean less K / V traffic, so: the
+    // largest of the three that still gives every one of the 256 CUs a workgroup.  256 queries run as
+    // sixteen wavefronts (8 query blocks x 2 key groups), the others as eight.  N_CTX need not divide.
     const int64_t ZH = dims[0], N = dims[1];
     block[0] = 512;
-    if (N > 0 && N % 256 == 0 && ZH > 0 && ZH <= 65535) {
+    if (N > 0 && N < (int64_t(1) << 24) && ZH > 0 && ZH <= 65535) {
       int64_t queries = 256;
-      while (queries > 64 && (N / queries) * ZH < 256)
+      while (queries > 64 && ((N + queries - 1) / queries) * ZH < 256)
         queries /= 2;
-      grid[0] = static_cast<size_t>(N / queries);
+      grid[0] = ceilDiv(N, queries);
       grid[1] = static_cast<size_t>(ZH);
       if (queries == 256)
         block[0] = 1024;

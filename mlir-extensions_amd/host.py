@@ -371,8 +371,8 @@ def input_fusion(stream, a, b, dtype="f32"):
 
 def flash_attention(stream, q, k, v, zh, n_ctx, sm_scale, queries_per_workgroup=None, threads=512):
     """WG/flash_attention_fwd.mlir:25-307: softmax(sm_scale * Q K^T) V per (batch, head);
-    q, k, v f16 bit patterns [(zh * n_ctx), 64].  `queries_per_workgroup` (64, 128 or 256,
-    n_ctx a multiple of 256) picks the tiling instead of the catalogue; 256 queries also come
+    q, k, v f16 bit patterns [(zh * n_ctx), 64].  `queries_per_workgroup` (64, 128 or 256)
+    picks the tiling instead of the catalogue; 256 queries also come
     with `threads` = 1024 (sixteen wavefronts, two key groups)."""
     for t in (q, k, v):
         _check(t, "f16")
@@ -383,11 +383,11 @@ def flash_attention(stream, q, k, v, zh, n_ctx, sm_scale, queries_per_workgroup=
     try:
         grid = block = None
         if queries_per_workgroup is not None:
-            if queries_per_workgroup not in (64, 128, 256) or n_ctx % 256:
-                raise ValueError("queries_per_workgroup must be 64, 128 or 256 and n_ctx a multiple of 256")
+            if queries_per_workgroup not in (64, 128, 256):
+                raise ValueError("queries_per_workgroup must be 64, 128 or 256")
             if threads not in (512, 1024) or (threads == 1024 and queries_per_workgroup != 256):
                 raise ValueError("threads is 512, or 1024 with 256 queries per workgroup")
-            grid, block = (n_ctx // queries_per_workgroup, zh, 1), (threads, 1, 1)
+            grid, block = (-(-n_ctx // queries_per_workgroup), zh, 1), (threads, 1, 1)
         stream.launch("imex_flash_attention_fwd_f16", [zh, n_ctx], [d_q, d_k, d_v, d_o, float(sm_scale), zh, n_ctx],
                       grid=grid, block=block)
         stream.wait()

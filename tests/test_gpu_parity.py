@@ -423,6 +423,48 @@ def test_flash_attention_every_tiling(host, orc, stream, zh, n_ctx, scale):
         assert attention_close(got[rows], ref, orc), (queries, threads)
 
 
+@pytest.mark.parametrize("zh,n_ctx,scale", [(2, 100, 0.5), (3, 1000, 0.125), (2, 257, 1.0), (1, 5, 0.5), (5, 333, 2.0),
+                                             (1, 193, 0.5), (2, 64, 0.5)])
+def test_flash_attention_ragged_context(host, orc, stream, zh, n_ctx, scale):
+    """N_CTX that divides none of the tiles: padded queries are not stored, padded keys get a
+    score of -inf; key groups that see no key at all (short heads) merge as empty.  Every
+    tiling, every row, against the oracle; the rows behind Out stay untouched."""
+    n = zh * n_ctx
+    q = orc.fill_uniform(n * 64, "f16", 81, -2, 2).reshape(n, 64)
+    k = orc.fill_uniform(n * 64, "f16", 82, -2, 2).reshape(n, 64)
+    v = orc.fill_uniform(n * 64, "f16", 83, -1, 1).reshape(n, 64)
+    rows = np.arange(n) if n <= 1200 else np.unique(np.concatenate([np.arange(0, n, 3), [n_ctx - 1, n_ctx, n - 1]]))
+    ref = orc.flash_attention_rows(q, k, v, n_ctx, scale, rows)
+    got = host.flash_attention(stream, q, k, v, zh, n_ctx, scale)
+    assert attention_close(got[rows], ref, orc), "catalogue launch"
+    for queries, threads in ((64, 512), (128, 512), (256, 512), (256, 1024)):
+        say("attention %dx%d ragged, %d queries per workgroup of %d threads" % (zh, n_ctx, queries, threads))
+        guard = np.full((n + 256, 64), 0x7e01, np.uint16)
+        d_q, d_k, d_v, d_o = (stream.to_device(t) for t in (q, k, v, guard))
+        grid = (-(-n_ctx // queries), zh, 1)
+        stream.launch("imex_flash_attention_fwd_f16", [zh, n_ctx], [d_q, d_k, d_v, d_o, float(scale), zh, n_ctx],
+                      grid=grid, block=(threads, 1, 1))
+        stream.wait()
+        out = stream.from_device(d_o, (n + 256, 64), np.uint16)
+        for p in (d_q, d_k, d_v, d_o):
+            stream.free(p)
+        assert np.all(out[n:] == 0x7e01), (queries, threads, "wrote behind Out")
+        assert attention_close(out[rows], ref, orc), (queries, threads)
+
+
+def test_flash_attention_negative_scale_takes_the_reference_loop(host, orc, stream):
+    """The tiled path takes the row maximum before scaling, which needs a positive scale; any
+    other scale runs the one-lane-per-query loop of the same kernel."""
+    zh, n_ctx = 2, 256
+    n = zh * n_ctx
+    q = orc.fill_uniform(n * 64, "f16", 84, -1, 1).reshape(n, 64)
+    k = orc.fill_uniform(n * 64, "f16", 85, -1, 1).reshape(n, 64)
+    v = orc.fill_uniform(n * 64, "f16", 86, -1, 1).reshape(n, 64)
+    rows = np.arange(0, n, 3)
+    got = host.flash_attention(stream, q, k, v, zh, n_ctx, -0.5)
+    assert attention_close(got[rows], orc.flash_attention_rows(q, k, v, n_ctx, -0.5, rows), orc)
+
+
 @pytest.mark.parametrize("zh", [8, 16])
 def test_flash_attention_catalogue_picks_wide_tilings(host, orc, stream, zh):
     """N_CTX = 4096 with 8 and 16 heads: the catalogue launches 128- and 256-query workgroups

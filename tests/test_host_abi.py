@@ -96,7 +96,9 @@ def test_launch_shapes(host):
     assert ls("imex_gemm_f16_f16_f32_tb", [256, 32768, 32768])[0] == (128, 1, 1)
     assert ls("imex_gemm_4kx4kx4k_f16_f16_f32", []) == ((16, 16, 1), (512, 1, 1), 0)
     assert ls("imex_flash_attention_fwd_f16", [4, 4096]) == ((64, 4, 1), (512, 1, 1), 0)
-    assert ls("imex_flash_attention_fwd_f16", [2, 100])[0] == (1, 1, 1)
+    assert ls("imex_flash_attention_fwd_f16", [2, 100])[0] == (2, 2, 1)    # N_CTX need not divide the tiles
+    assert ls("imex_flash_attention_fwd_f16", [40, 1000])[:2] == ((8, 40, 1), (512, 1, 1))
+    assert ls("imex_flash_attention_fwd_f16", [64, 1000])[:2] == ((4, 64, 1), (1024, 1, 1))
     # 64, 128 or 256 queries per workgroup: the most that still leaves 256 workgroups
     assert ls("imex_flash_attention_fwd_f16", [8, 4096])[0] == (32, 8, 1)
     assert ls("imex_flash_attention_fwd_f16", [16, 4096])[:2] == ((16, 16, 1), (1024, 1, 1))  # 256 queries: 16 wavefronts
