@@ -124,6 +124,19 @@ std::vector<Workload> workloads() {
       {"transpose3d_f32_16x96x96", "imex_transpose3d_b32", {16, 96, 96},
        {{Elem::F32, {16, 96, 96}, true, -1, 1}, {Elem::F32, {96, 96, 16}, false, 0, 0}}, {16, 96, 96}, 0,
        2.0 * 16 * 96 * 96 * 4, false},
+      // the fused chains at the benchmark's own size (launch-bound) and at one that streams from HBM
+      {"loop_fusion_f32_512x1024", "imex_loop_fusion_f32", {512 * 1024},
+       {{Elem::F32, {512 * 1024}, true, 0.5f, 3}, {Elem::F32, {512 * 1024}, true, -3, 3},
+        {Elem::F32, {512 * 1024}, false, 0, 0}}, {512 * 1024}, 0, 3.0 * 512 * 1024 * 4, false},
+      {"loop_fusion_f32_4096x4096", "imex_loop_fusion_f32", {K4 * K4},
+       {{Elem::F32, {K4 * K4}, true, 0.5f, 3}, {Elem::F32, {K4 * K4}, true, -3, 3}, {Elem::F32, {K4 * K4}, false, 0, 0}},
+       {K4 * K4}, 0, 3.0 * K4 * K4 * 4, false},
+      {"input_fusion_f32_512x1024", "imex_input_fusion_f32", {512, 1024},
+       {{Elem::F32, {512, 1024}, true, -3, 3}, {Elem::F32, {512, 1024}, true, 0.5f, 3}, {Elem::F32, {1024}, false, 0, 0}},
+       {512, 1024}, 0, 2.0 * 512 * 1024 * 4 + 1024 * 4, false},
+      {"input_fusion_f32_8192x8192", "imex_input_fusion_f32", {K8, K8},
+       {{Elem::F32, {K8, K8}, true, -3, 3}, {Elem::F32, {K8, K8}, true, 0.5f, 3}, {Elem::F32, {K8}, false, 0, 0}},
+       {K8, K8}, 0, 2.0 * K8 * K8 * 4 + K8 * 4, false},
       // not operators: the MFMA pipe fed from LDS with nothing else going on, one workgroup per CU,
       // on hashed f16 operands in (-1,1) and on zeros -- the rate the GEMMs' operand values allow
       {"mfma_lds_ceiling_f16_random", "imex_mfma_lds_ceiling_f16", {256 * 512},

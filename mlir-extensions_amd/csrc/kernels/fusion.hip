@@ -20,7 +20,8 @@
 // Arguments:  loop fusion  (a, b, out, n: i64)              dims = {n}
 //             input fusion (a, b, out, rows: i64, cols: i64) dims = {rows, cols}
 // Launch: block (256,1,1); loop fusion grid ceil(n / 4096) (f32) or ceil(n / 8192)
-// (16-bit); input fusion grid ceil(cols / 256), one thread per output column.
+// (16-bit); input fusion grid ceil(cols / c), a workgroup per block of c = 64 .. 4 columns
+// (the widest that leaves 512 workgroups).  Workgroups stride, so any grid is correct.
 
 #include "device_common.h"
 
@@ -180,33 +181,81 @@ __device__ __forceinline__ void loop_fusion(const void *__restrict__ a, const vo
 }
 
 // ---- kInputFusion: chain + column sums ------------------------------------------------
-// One thread per output column, rows added in ascending order from +0.0 -- the
-// reference's order, so the f32 result is the same bits.  Consecutive lanes read
-// consecutive columns (coalesced); eight rows of loads are in flight per lane.
+// out[j] = sum over rows i, in ascending order from +0.0, of chain(a[i,j], b[i,j]) -- the
+// reference's order of additions, so the f32 result is the same bits.  Only the additions are
+// ordered; the chain (a logarithm per element) is not.  A workgroup owns kCols adjacent columns
+// and walks the rows in tiles of 4096 / kCols: all 256 lanes evaluate the chain of a tile into
+// LDS (coalesced along the rows), then lane j < kCols adds column j's values of the tile to its
+// running sum, in row order.  The tile is double-buffered, so the ordered additions of one tile
+// run under the loads and logarithms of the next, with one barrier per tile.
+constexpr int kTileElems = 4096;
+
+template <Dt D, int kCols>
+__device__ __forceinline__ void input_fusion_cols(const void *__restrict__ a, const void *__restrict__ b,
+                                                  void *__restrict__ out, int64_t rows, int64_t cols,
+                                                  const LogfEntry *table, float *tile) {
+  using E = Elem<D>;
+  constexpr int kTileRows = kTileElems / kCols;
+  constexpr int kPerLane = kTileElems / kThreads;
+  const int tid = threadIdx.x;
+  for (int64_t c0 = int64_t(blockIdx.x) * kCols; c0 < cols; c0 += int64_t(gridDim.x) * kCols) {
+    float acc = 0.0f;
+    int buf = 0;
+    for (int64_t r0 = 0; r0 < rows; r0 += kTileRows, buf ^= 1) {
+      float *t = tile + buf * kTileElems;
+      float xa[kPerLane], xb[kPerLane];
+#pragma unroll
+      for (int u = 0; u < kPerLane; ++u) {
+        const int e = u * kThreads + tid;
+        const int64_t r = r0 + e / kCols, c = c0 + e % kCols;
+        const bool ok = r < rows && c < cols;
+        xa[u] = ok ? E::get(a, r * cols + c) : 1.0f;
+        xb[u] = ok ? E::get(b, r * cols + c) : 1.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < kPerLane; ++u)
+        t[u * kThreads + tid] = input_chain(xa[u], xb[u], table);
+      __syncthreads(); // the tile is complete; the other buffer was consumed before the previous barrier
+      if (tid < kCols && c0 + tid < cols) {
+        const int n = rows - r0 < kTileRows ? int(rows - r0) : kTileRows;
+        int r = 0;
+        for (; r + 16 <= n; r += 16) { // sixteen LDS reads in flight, then the additions in row order
+          float v[16];
+#pragma unroll
+          for (int u = 0; u < 16; ++u)
+            v[u] = t[(r + u) * kCols + tid];
+#pragma unroll
+          for (int u = 0; u < 16; ++u)
+            acc = acc + v[u];
+        }
+        for (; r < n; ++r)
+          acc = acc + t[r * kCols + tid];
+      }
+    }
+    if (tid < kCols && c0 + tid < cols)
+      E::put(out, c0 + tid, acc);
+    __syncthreads(); // both buffers are free for the next block of columns
+  }
+}
+
+// Columns per workgroup: as many as still leave every CU a couple of workgroups (wide blocks read
+// longer row segments), down to 4.
+__device__ __forceinline__ int input_fusion_block_cols(int64_t cols) {
+  return cols >= 64 * 512 ? 64 : cols >= 32 * 512 ? 32 : cols >= 16 * 512 ? 16 : cols >= 8 * 512 ? 8 : 4;
+}
+
 template <Dt D>
 __device__ __forceinline__ void input_fusion(const void *__restrict__ a, const void *__restrict__ b,
                                              void *__restrict__ out, int64_t rows, int64_t cols) {
-  using E = Elem<D>;
   __shared__ LogfEntry table[16];
+  __shared__ float tile[2 * kTileElems];
   stage_table(table);
-  const int64_t stride = int64_t(gridDim.x) * kThreads;
-  for (int64_t col = int64_t(blockIdx.x) * kThreads + threadIdx.x; col < cols; col += stride) {
-    float acc = 0.0f;
-    int64_t i = 0;
-    for (; i + 8 <= rows; i += 8) {
-      float xa[8], xb[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        xa[u] = E::get(a, (i + u) * cols + col);
-        xb[u] = E::get(b, (i + u) * cols + col);
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        acc = acc + input_chain(xa[u], xb[u], table);
-    }
-    for (; i < rows; ++i)
-      acc = acc + input_chain(E::get(a, i * cols + col), E::get(b, i * cols + col), table);
-    E::put(out, col, acc);
+  switch (input_fusion_block_cols(cols)) {
+  case 64: input_fusion_cols<D, 64>(a, b, out, rows, cols, table, tile); break;
+  case 32: input_fusion_cols<D, 32>(a, b, out, rows, cols, table, tile); break;
+  case 16: input_fusion_cols<D, 16>(a, b, out, rows, cols, table, tile); break;
+  case 8: input_fusion_cols<D, 8>(a, b, out, rows, cols, table, tile); break;
+  default: input_fusion_cols<D, 4>(a, b, out, rows, cols, table, tile); break;
   }
 }
 

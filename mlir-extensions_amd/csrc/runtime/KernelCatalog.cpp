@@ -218,9 +218,12 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     }
     break;
   }
-  case Shape::ColumnThreads: // one lane per output column
-    grid[0] = ceilDiv(dims[1], 256);
+  case Shape::ColumnThreads: { // a workgroup per block of 64 .. 4 columns: the widest that leaves 512 workgroups
+    const int64_t cols = dims[1];
+    const int64_t block_cols = cols >= 64 * 512 ? 64 : cols >= 32 * 512 ? 32 : cols >= 16 * 512 ? 16 : cols >= 8 * 512 ? 8 : 4;
+    grid[0] = ceilDiv(cols, block_cols);
     break;
+  }
   case Shape::Gemm:
   case Shape::GemmTA:
   case Shape::GemmTB: {

@@ -104,7 +104,8 @@ def test_launch_shapes(host):
     assert ls("imex_flash_attention_fwd_f16", [16, 4096])[:2] == ((16, 16, 1), (1024, 1, 1))  # 256 queries: 16 wavefronts
     assert ls("imex_flash_attention_fwd_f16", [64, 1024])[:2] == ((4, 64, 1), (1024, 1, 1))
     assert ls("imex_flash_attention_fwd_f16", [3, 256])[0] == (4, 3, 1)
-    assert ls("imex_input_fusion_f32", [512, 1024])[0] == (4, 1, 1)
+    assert ls("imex_input_fusion_f32", [512, 1024])[0] == (256, 1, 1)      # 4 columns per workgroup
+    assert ls("imex_input_fusion_f32", [512, 65536])[0] == (1024, 1, 1)    # 64
     assert ls("imex_gemm_4kx4kx4k_transpose_a", []) == ((16, 16, 1), (512, 1, 1), 0)
     assert ls("imex_gemm_f16_f16_f32_tb", [512, 256, 96])[0] == (2, 1, 1)
     assert ls("imex_mfma_lds_ceiling_f16", [256 * 512]) == ((256, 1, 1), (512, 1, 1), 0)
@@ -308,7 +309,7 @@ def test_launch_shapes_cover_the_problem(host):
         (gx, _, _), _, _ = ls("imex_reduce_outer_f32", [rows, cols])
         assert gx >= 1 and gx * 8192 >= cols  # the kernel strides over whatever the grid leaves
         (gx, _, _), _, _ = ls("imex_input_fusion_f32", [rows, cols])
-        assert gx * 256 >= cols
+        assert gx * 64 >= cols
         (gx, _, _), _, _ = ls("imex_softmax_f16", [rows, cols])
         assert gx >= 1 and (gx * 4 >= rows if cols <= 1024 else gx >= min(rows, 1048560))
 
