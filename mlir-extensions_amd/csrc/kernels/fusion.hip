@@ -20,7 +20,7 @@
 // Arguments:  loop fusion  (a, b, out, n: i64)              dims = {n}
 //             input fusion (a, b, out, rows: i64, cols: i64) dims = {rows, cols}
 // Launch: block (256,1,1); loop fusion grid ceil(n / 4096) (f32) or ceil(n / 8192)
-// (16-bit); input fusion grid ceil(cols / c), a workgroup per block of c = 64 .. 4 columns
+// (16-bit), a quarter of that per workgroup below 4 Mi elements; input fusion grid ceil(cols / c), a workgroup per block of c = 64 .. 4 columns
 // (the widest that leaves 512 workgroups).  Workgroups stride, so any grid is correct.
 
 #include "device_common.h"
@@ -30,7 +30,6 @@ using namespace imexhip;
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kVecsPerThread = 4;
 
 // ---------------------------------------------------------------------------
 // logf as glibc computes it (Arm Optimized Routines logf: x = 2^k z with z in
@@ -142,12 +141,16 @@ template <> struct Elem<Dt::F16> : Elem16<false> {};
 template <> struct Elem<Dt::BF16> : Elem16<true> {};
 
 // ---- kLoopFusion: two streams in, one out ------------------------------------------
-template <Dt D>
-__device__ __forceinline__ void loop_fusion(const void *__restrict__ a, const void *__restrict__ b,
-                                            void *__restrict__ out, int64_t n) {
+// kVecs 16-byte vectors per lane and pass: four for tensors that stream from HBM, one for small
+// ones, where the logarithms of a lane are the critical path and spreading them over more
+// workgroups is what shortens it.
+constexpr int64_t kSmallFusion = int64_t(1) << 22; // elements
+
+template <Dt D, int kVecs>
+__device__ __forceinline__ void loop_fusion_pass(const void *__restrict__ a, const void *__restrict__ b,
+                                                 void *__restrict__ out, int64_t n, const LogfEntry *table) {
   using E = Elem<D>;
-  __shared__ LogfEntry table[16];
-  stage_table(table);
+  constexpr int kVecsPerThread = kVecs;
   constexpr int64_t kElemsPerBlock = int64_t(kThreads) * kVecsPerThread * E::kPerVec;
   const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
                          reinterpret_cast<uintptr_t>(out)) & 15) == 0;
@@ -178,6 +181,17 @@ __device__ __forceinline__ void loop_fusion(const void *__restrict__ a, const vo
         E::put(out, i, loop_chain(E::get(a, i), E::get(b, i), table));
     }
   }
+}
+
+template <Dt D>
+__device__ __forceinline__ void loop_fusion(const void *__restrict__ a, const void *__restrict__ b,
+                                            void *__restrict__ out, int64_t n) {
+  __shared__ LogfEntry table[16];
+  stage_table(table);
+  if (n < kSmallFusion)
+    loop_fusion_pass<D, 1>(a, b, out, n, table);
+  else
+    loop_fusion_pass<D, 4>(a, b, out, n, table);
 }
 
 // ---- kInputFusion: chain + column sums ------------------------------------------------
@@ -214,16 +228,29 @@ __device__ __forceinline__ void input_fusion_cols(const void *__restrict__ a, co
       }
 #pragma unroll
       for (int u = 0; u < kPerLane; ++u)
-        t[u * kThreads + tid] = input_chain(xa[u], xb[u], table);
+        if (r0 + (u * kThreads) / kCols < rows) // uniform: passes that lie wholly below the last row are skipped
+          t[u * kThreads + tid] = input_chain(xa[u], xb[u], table);
       __syncthreads(); // the tile is complete; the other buffer was consumed before the previous barrier
       if (tid < kCols && c0 + tid < cols) {
         const int n = rows - r0 < kTileRows ? int(rows - r0) : kTileRows;
+        // sixteen LDS reads are in flight while the previous sixteen values are added in row order
+        float v[16], w[16];
         int r = 0;
-        for (; r + 16 <= n; r += 16) { // sixteen LDS reads in flight, then the additions in row order
-          float v[16];
+        if (n >= 16) {
 #pragma unroll
           for (int u = 0; u < 16; ++u)
-            v[u] = t[(r + u) * kCols + tid];
+            v[u] = t[u * kCols + tid];
+          for (r = 16; r + 16 <= n; r += 16) {
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+              w[u] = t[(r + u) * kCols + tid];
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+              acc = acc + v[u];
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+              v[u] = w[u];
+          }
 #pragma unroll
           for (int u = 0; u < 16; ++u)
             acc = acc + v[u];

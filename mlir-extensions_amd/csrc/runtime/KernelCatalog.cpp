@@ -28,7 +28,7 @@ extern const unsigned char imex_blob_probe[], imex_blob_probe_end[];
 namespace {
 
 enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm, Fusion, Attention, Probe };
-enum class Shape { Eltwise32, Eltwise16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, Attention, LanesOf512 };
+enum class Shape { Eltwise32, Eltwise16, Fusion32, Fusion16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, Attention, LanesOf512 };
 
 struct Entry {
   const char *name;
@@ -55,9 +55,9 @@ const Entry kEntries[] = {
      Shape::Transpose3D32, 3},
     {"imex_transpose3d_b16", "(in: b16*, out: b16*, d0: i64, d1: i64, d2: i64)", Module::Transpose,
      Shape::Transpose3D16, 3},
-    {"imex_loop_fusion_f32", "(a: f32*, b: f32*, out: f32*, n: i64)", Module::Fusion, Shape::Eltwise32, 1},
-    {"imex_loop_fusion_f16", "(a: f16*, b: f16*, out: f16*, n: i64)", Module::Fusion, Shape::Eltwise16, 1},
-    {"imex_loop_fusion_bf16", "(a: bf16*, b: bf16*, out: bf16*, n: i64)", Module::Fusion, Shape::Eltwise16, 1},
+    {"imex_loop_fusion_f32", "(a: f32*, b: f32*, out: f32*, n: i64)", Module::Fusion, Shape::Fusion32, 1},
+    {"imex_loop_fusion_f16", "(a: f16*, b: f16*, out: f16*, n: i64)", Module::Fusion, Shape::Fusion16, 1},
+    {"imex_loop_fusion_bf16", "(a: bf16*, b: bf16*, out: bf16*, n: i64)", Module::Fusion, Shape::Fusion16, 1},
     {"imex_input_fusion_f32", "(a: f32*, b: f32*, out: f32*, rows: i64, cols: i64)", Module::Fusion,
      Shape::ColumnThreads, 2},
     {"imex_input_fusion_f16", "(a: f16*, b: f16*, out: f16*, rows: i64, cols: i64)", Module::Fusion,
@@ -154,6 +154,12 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     break;
   case Shape::Eltwise16: // 256 lanes x 4 vectors x 8 elements
     grid[0] = ceilDiv(dims[0], 8192);
+    break;
+  case Shape::Fusion32: // as Eltwise32 / 16, but one vector per lane below 4 Mi elements
+    grid[0] = ceilDiv(dims[0], dims[0] < (int64_t(1) << 22) ? 1024 : 4096);
+    break;
+  case Shape::Fusion16:
+    grid[0] = ceilDiv(dims[0], dims[0] < (int64_t(1) << 22) ? 2048 : 8192);
     break;
   case Shape::SoftmaxRows32:
   case Shape::SoftmaxRows16: {

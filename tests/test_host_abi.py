@@ -295,8 +295,10 @@ def test_launch_shapes_cover_the_problem(host):
     @settings(max_examples=300, deadline=None)
     @given(n=st.integers(1, 1 << 34))
     def eltwise(n):
+        small = n < (1 << 22)
         for name, per in (("imex_relu_f32", 4096), ("imex_silu_f32", 4096), ("imex_relu_bf16", 8192),
-                          ("imex_loop_fusion_f32", 4096), ("imex_loop_fusion_f16", 8192)):
+                          ("imex_loop_fusion_f32", 1024 if small else 4096),
+                          ("imex_loop_fusion_f16", 2048 if small else 8192)):
             (gx, gy, gz), block, _ = ls(name, [n])
             assert block == (256, 1, 1) and gy == gz == 1
             assert (gx - 1) * per < n <= gx * per
