@@ -237,6 +237,48 @@ def measure_rotating(host, stream, w, passes):
     return ms, copies
 
 
+def measure_reference_suite(stream):
+    """Every shape and dtype the reference's benchmark suite instantiates (README.md:330-335, benchmarks/*/
+    *.shapes.in, *.dtypes.in) plus the two fused chains at their size (512x1024): microseconds per launch over 200
+    back-to-back launches on zero-filled buffers.  Most of them are launch-bound (2.5-4 us)."""
+    out = {}
+
+    def run(label, kernel, dims, sizes, scalars):
+        ptrs = [stream.alloc(n) for n in sizes]
+        ms = stream.profile(kernel, dims, ptrs + scalars, warmups=20, rounds=200, mode=1)[0] / 200
+        for p in ptrs:
+            stream.free(p)
+        out[label] = round(ms * 1e3, 2)
+
+    width = {"f32": 4, "f16": 2, "bf16": 2}
+    for shape in ((1, 160, 160, 120), (50, 640, 20, 15), (512, 640, 20, 15)):
+        n = int(np.prod(shape))
+        for dt, w in width.items():
+            run("relu_%s_%s" % (dt, "x".join(map(str, shape))), "imex_relu_" + dt, [n], [n * w, n * w], [n])
+    for shape in ((1, 1024, 40, 30), (50, 20, 3072), (512, 640, 20, 15)):
+        n = int(np.prod(shape))
+        run("silu_f32_%s" % "x".join(map(str, shape)), "imex_silu_f32", [n], [n * 4, n * 4], [n])
+    for rows in (1, 16, 64, 256, 1024):
+        for dt, w in width.items():
+            n = rows * 2000
+            run("softmax_%s_%dx2000" % (dt, rows), "imex_softmax_" + dt, [rows, 2000], [n * w, n * w], [rows, 2000])
+    for r, c in ((128, 136), (1024, 1024)):
+        for bits in (32, 16):
+            n = r * c * bits // 8
+            run("transpose_b%d_%dx%d" % (bits, r, c), "imex_transpose2d_b%d" % bits, [r, c], [n, n], [r, c])
+    for d in ((16, 96, 96), (96, 7, 96)):
+        for bits in (32, 16):
+            n = d[0] * d[1] * d[2] * bits // 8
+            run("transpose_b%d_%dx%dx%d" % ((bits,) + d), "imex_transpose3d_b%d" % bits, list(d), [n, n], list(d))
+    inner = 16 * 512 * 512
+    run("reduce_f32_32x16x512x512", "imex_reduce_outer_f32", [32, inner], [32 * inner * 4, inner * 4], [32, inner, 0.0])
+    for dt, w in width.items():
+        n = 512 * 1024
+        run("loop_fusion_%s_512x1024" % dt, "imex_loop_fusion_" + dt, [n], [n * w] * 3, [n])
+        run("input_fusion_%s_512x1024" % dt, "imex_input_fusion_" + dt, [512, 1024], [n * w, n * w, 1024 * w], [512, 1024])
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -244,6 +286,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--only", type=str, default=None, help="comma-separated workload names")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline legs")
+    ap.add_argument("--suite", action="store_true",
+                    help="also time every shape of the reference's benchmark suite (us per launch, back to back)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every kernel here runs on a single MI355X and this build has no "
@@ -362,6 +406,9 @@ def main():
             entry_["cpu_baseline"] = {"value": round(v, 6), "unit": w.unit, "cores": 1, "kind": "port", "sample": sample}
             log("cpu baseline %s: %.4f %s (%.1f s)" % (w.name, v, w.unit, time.time() - t))
     result["per_config"] = per
+    if args.suite:
+        result["reference_suite_us_per_launch"] = measure_reference_suite(stream)
+        log("reference benchmark suite: %d shapes timed" % len(result["reference_suite_us_per_launch"]))
 
     for w in workloads:
         for p in w.buffers:

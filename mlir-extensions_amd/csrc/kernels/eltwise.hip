@@ -17,13 +17,12 @@ using namespace imexhip;
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kVecsPerThread = 4; // 4 x 16 B per lane in flight
 
 // ---------------------------------------------------------------------------
 // Generic streaming driver: Op works on one 16-byte vector (u32x4) and on one
 // scalar element (for ragged tails and unaligned bases).
 // ---------------------------------------------------------------------------
-template <typename Op, int kElemBytes, bool kStream>
+template <typename Op, int kElemBytes, bool kStream, int kVecsPerThread = 4>
 __device__ __forceinline__ void stream_map_impl(const void *__restrict__ in, void *__restrict__ out, int64_t n,
                                                 Op op) {
   constexpr int kElemsPerVec = 16 / kElemBytes;
@@ -182,5 +181,10 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_silu_f32(const float
   if (threadIdx.x < 32)
     table[threadIdx.x] = kExp2Table[threadIdx.x];
   __syncthreads();
-  stream_map<SiluF32, 4>(in, out, n, SiluF32{table});
+  // Below 4 Mi elements a lane's exponentials and divisions are the critical path: one vector
+  // per lane and pass (four times the workgroups) instead of four.
+  if (n < (int64_t(1) << 22))
+    stream_map_impl<SiluF32, 4, true, 1>(in, out, n, SiluF32{table});
+  else
+    stream_map<SiluF32, 4>(in, out, n, SiluF32{table});
 }

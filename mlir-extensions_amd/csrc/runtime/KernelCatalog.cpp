@@ -42,7 +42,7 @@ const Entry kEntries[] = {
     {"imex_relu_f32", "(in: f32*, out: f32*, n: i64)", Module::Eltwise, Shape::Eltwise32, 1},
     {"imex_relu_f16", "(in: f16*, out: f16*, n: i64)", Module::Eltwise, Shape::Eltwise16, 1},
     {"imex_relu_bf16", "(in: bf16*, out: bf16*, n: i64)", Module::Eltwise, Shape::Eltwise16, 1},
-    {"imex_silu_f32", "(in: f32*, out: f32*, n: i64)", Module::Eltwise, Shape::Eltwise32, 1},
+    {"imex_silu_f32", "(in: f32*, out: f32*, n: i64)", Module::Eltwise, Shape::Fusion32, 1},
     {"imex_softmax_f32", "(in: f32*, out: f32*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows32, 2},
     {"imex_softmax_f16", "(in: f16*, out: f16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows16, 2},
     {"imex_softmax_bf16", "(in: bf16*, out: bf16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows16, 2},
@@ -155,7 +155,7 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
   case Shape::Eltwise16: // 256 lanes x 4 vectors x 8 elements
     grid[0] = ceilDiv(dims[0], 8192);
     break;
-  case Shape::Fusion32: // as Eltwise32 / 16, but one vector per lane below 4 Mi elements
+  case Shape::Fusion32: // SiLU and the fused chains: as Eltwise32 / 16, but one vector per lane below 4 Mi elements
     grid[0] = ceilDiv(dims[0], dims[0] < (int64_t(1) << 22) ? 1024 : 4096);
     break;
   case Shape::Fusion16:

@@ -296,7 +296,7 @@ def test_launch_shapes_cover_the_problem(host):
     @given(n=st.integers(1, 1 << 34))
     def eltwise(n):
         small = n < (1 << 22)
-        for name, per in (("imex_relu_f32", 4096), ("imex_silu_f32", 4096), ("imex_relu_bf16", 8192),
+        for name, per in (("imex_relu_f32", 4096), ("imex_silu_f32", 1024 if small else 4096), ("imex_relu_bf16", 8192),
                           ("imex_loop_fusion_f32", 1024 if small else 4096),
                           ("imex_loop_fusion_f16", 2048 if small else 8192)):
             (gx, gy, gz), block, _ = ls(name, [n])
