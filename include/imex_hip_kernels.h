@@ -21,6 +21,8 @@
  *       benchmarks/softmax/softmax_gpu.mlir.in:4-44      dims = {rows, cols}
  *   imex_rowsum_f32                (in, out, rows:i64, cols:i64, init:f32)
  *       WG/reduction_2D_1D_cross_sg_cross_lane.mlir:31-37 dims = {rows, cols}
+ *   imex_rowmean_f32               (in, out, rows:i64, cols:i64)   out[r] = (sum_c in[r,c]) / cols
+ *       WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir:51-52   dims = {rows, cols}
  *   imex_reduce_outer_f32          (in, out, outer:i64, inner:i64, init:f32)
  *       benchmarks/reduce/reduce_gpu.mlir.in:4-21        dims = {outer, inner}
  *   imex_transpose2d_b16 / _b32    (in, out, rows:i64, cols:i64)

@@ -12,7 +12,11 @@
 //    owns groups of four adjacent outputs and adds the `outer` slices in order,
 //    which is the reference's summation order, so this one is bit-exact.
 //
-// Arguments: rowsum (in, out, rows: i64, cols: i64, init: f32);
+//  * imex_rowmean_f32: out[r] = (0 + sum_c in[r, c]) / cols, the same reduction with the
+//    division the reference applies afterwards
+//    (WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir:51-52, 1x24x1024x64 -> 1x24x1024x1).
+//
+// Arguments: rowsum (in, out, rows: i64, cols: i64, init: f32); rowmean (in, out, rows: i64, cols: i64);
 //            reduce_outer (in, out, outer: i64, inner: i64, init: f32).
 // Launch: block (256,1,1);
 //   rowsum: cols > 2048 -> grid (rows,1,1) [workgroup per row],
@@ -71,8 +75,11 @@ __device__ __forceinline__ float row_partial(const float *__restrict__ row, int6
 
 } // namespace
 
-extern "C" __global__ __launch_bounds__(kThreads) void imex_rowsum_f32(const float *in, float *out, int64_t rows,
-                                                                      int64_t cols, float init) {
+// kMean: the sum (from `init`) divided by the row length, the post-op of
+// WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir:51-52.
+template <bool kMean>
+__device__ __forceinline__ void row_reduce(const float *in, float *out, int64_t rows, int64_t cols, float init) {
+  const float divisor = static_cast<float>(cols);
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   // the input is read exactly once: stream it past the caches (non-temporal)
@@ -88,7 +95,8 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_rowsum_f32(const flo
         partial[wave] = s;
       __syncthreads();
       if (threadIdx.x == 0)
-        out[row] = init + ((partial[0] + partial[1]) + (partial[2] + partial[3]));
+        out[row] = kMean ? (init + ((partial[0] + partial[1]) + (partial[2] + partial[3]))) / divisor
+                         : init + ((partial[0] + partial[1]) + (partial[2] + partial[3]));
       __syncthreads(); // `partial` is reused by the next row
     }
   } else {
@@ -98,9 +106,19 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_rowsum_f32(const flo
                              : row_partial<false>(in + row * cols, cols, lane, kWave);
       float s = wave_sum(p);
       if (lane == 0)
-        out[row] = init + s;
+        out[row] = kMean ? (init + s) / divisor : init + s;
     }
   }
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_rowsum_f32(const float *in, float *out, int64_t rows,
+                                                                      int64_t cols, float init) {
+  row_reduce<false>(in, out, rows, cols, init);
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_rowmean_f32(const float *in, float *out, int64_t rows,
+                                                                       int64_t cols) {
+  row_reduce<true>(in, out, rows, cols, 0.0f);
 }
 
 // Outer-dimension sum: lane owns kVecs vectors of four adjacent outputs, 4 KiB apart, so a

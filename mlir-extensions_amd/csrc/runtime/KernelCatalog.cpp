@@ -47,6 +47,7 @@ const Entry kEntries[] = {
     {"imex_softmax_f16", "(in: f16*, out: f16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows16, 2},
     {"imex_softmax_bf16", "(in: bf16*, out: bf16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows16, 2},
     {"imex_rowsum_f32", "(in: f32*, out: f32*, rows: i64, cols: i64, init: f32)", Module::Reduce, Shape::RowSum, 2},
+    {"imex_rowmean_f32", "(in: f32*, out: f32*, rows: i64, cols: i64)", Module::Reduce, Shape::RowSum, 2},
     {"imex_reduce_outer_f32", "(in: f32*, out: f32*, outer: i64, inner: i64, init: f32)", Module::Reduce,
      Shape::ReduceOuter, 2},
     {"imex_transpose2d_b32", "(in: b32*, out: b32*, rows: i64, cols: i64)", Module::Transpose, Shape::Transpose2D32, 2},

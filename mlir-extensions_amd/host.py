@@ -422,6 +422,12 @@ def rowsum(stream, x, init=0.0):
     return _unary(stream, "imex_rowsum_f32", x, "f32", [rows, cols], extra=[float(init)], out_shape=(rows,))
 
 
+def rowmean(stream, x):
+    """WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir:51-52: mean over the last dimension."""
+    rows, cols = x.shape
+    return _unary(stream, "imex_rowmean_f32", x, "f32", [rows, cols], out_shape=(rows,))
+
+
 def reduce_outer(stream, x, init=0.0):
     """benchmarks/reduce/reduce_gpu.mlir.in:4-21: the outermost dim is summed away."""
     outer = x.shape[0]

@@ -402,6 +402,18 @@ void oracle_rowsum_f32(const float *x, float *out, int64_t rows, int64_t cols, f
   }
 }
 
+/* WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir:115-127: the sequential sum from 0 over the last
+   dimension, then one arith.divf by the dimension's length. */
+void oracle_rowmean_f32(const float *x, float *out, int64_t rows, int64_t cols) {
+  const float n = (float)cols;
+  for (int64_t r = 0; r < rows; ++r) {
+    float acc = 0.0f;
+    const float *xr = x + r * cols;
+    for (int64_t c = 0; c < cols; ++c) acc = acc + xr[c];
+    out[r] = acc / n;
+  }
+}
+
 /* benchmarks/reduce/reduce_gpu.mlir.in:4-21: in is [outer, inner...] and the
    OUTERMOST dimension is reduced: out[i] = init; for d3: out[i] = out[i] + in[d3, i]. */
 void oracle_reduce_outer_f32(const float *x, float *out, int64_t outer, int64_t inner, float init) {

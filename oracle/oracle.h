@@ -84,6 +84,7 @@ void oracle_softmax_16(const uint16_t *x, uint16_t *y, int64_t rows, int64_t col
 
 /* ---- reductions ------------------------------------------------------------ */
 void oracle_rowsum_f32(const float *x, float *out, int64_t rows, int64_t cols, float init);       /* WG/reduction_2D_1D_cross_sg_cross_lane.mlir:31-37 */
+void oracle_rowmean_f32(const float *x, float *out, int64_t rows, int64_t cols);                      /* WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir:115-127 */
 void oracle_reduce_outer_f32(const float *x, float *out, int64_t outer, int64_t inner, float init); /* benchmarks/reduce/reduce_gpu.mlir.in:4-21 */
 float oracle_sum_all_f32(const float *x, int64_t n, float init);                                   /* test/PlaidML/OpTest.Sum.mlir:18-26 */
 

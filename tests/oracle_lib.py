@@ -223,6 +223,13 @@ def rowsum_f32(x, init=0.0):
     return out
 
 
+def rowmean_f32(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape[0], np.float32)
+    lib().oracle_rowmean_f32(_p(x), _p(out), C.c_int64(x.shape[0]), C.c_int64(x.shape[1]))
+    return out
+
+
 def reduce_outer_f32(x, init=0.0):
     x = _c(x, np.float32)
     outer = x.shape[0]

@@ -171,6 +171,19 @@ def test_rowsum_config_8192x8192(host, orc, stream):
     assert np.max(np.abs(got - exact) / exact) < 1e-5
 
 
+def test_rowmean(host, orc, stream):
+    """Mean over the last dimension (WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir: 1x24x1024x64,
+    uniform(-1,1) inputs, checked there against the sequential CPU loop with allclose)."""
+    x = orc.fill_uniform(24 * 1024 * 64, "f32", 79, -1.0, 1.0).reshape(24 * 1024, 64)
+    got, ref = host.rowmean(stream, x), orc.rowmean_f32(x)
+    assert np.all(np.abs(got - ref) <= 1e-4 + 1e-3 * np.abs(ref))   # the reference's allclose
+    assert np.max(np.abs(got - ref)) <= 2e-7                          # and far inside it
+    # integer-valued rows: the sum is exact in any order, so the mean is the oracle's bits
+    for rows, cols in ((7, 64), (5, 3000), (1000, 96), (3, 1)):
+        m = orc.fill_int(rows * cols, "f32", 80, -8, 8).reshape(rows, cols)
+        assert np.array_equal(host.rowmean(stream, m), orc.rowmean_f32(m)), (rows, cols)
+
+
 @pytest.mark.parametrize("shape", [(32, 16, 64, 64), (10, 20), (7, 1023), (33, 4100), (1, 5), (3, 1, 9),
                                    (5, 512 * 2048 + 4), (3, 512 * 4096 + 1028), (2, 512 * 8192 + 8), (6, 512 * 2048 + 3)])
 def test_reduce_outer_bit_exact(host, orc, stream, shape):

@@ -308,6 +308,23 @@ def test_rowsum_is_sequential(orc):
     assert orc.rowsum_f32(np.ones((1, 3), np.float32), init=2.5)[0] == 5.5
 
 
+def test_rowmean_closed_forms(orc):
+    """WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir:115-127: sequential sum, then one division.
+    Pinned by what arithmetic fixes: a constant dyadic row of a power-of-two length returns the constant
+    exactly; integers 0..63 average 31.5; the sum is sequential (2^24 absorbs ones added after it,
+    not before); the division is by the row length, not a multiplication by a rounded reciprocal."""
+    assert np.array_equal(orc.rowmean_f32(np.full((3, 64), 0.625, np.float32)), np.full(3, np.float32(0.625)))
+    assert orc.rowmean_f32(np.arange(64, dtype=np.float32)[None, :])[0] == np.float32(31.5)
+    big = np.concatenate([[np.float32(2 ** 24)], np.ones(63, np.float32)])[None, :]
+    assert orc.rowmean_f32(big)[0] == np.float32(2 ** 24) / np.float32(64)
+    assert orc.rowmean_f32(big[:, ::-1].copy())[0] == np.float32(2 ** 24 + 63) / np.float32(64)
+    x = np.array([[1.0, 2.0, 4.0]], np.float32)   # 7 / 3 correctly rounded differs from 7 * fl(1/3)
+    assert orc.rowmean_f32(x)[0] == np.float32(7.0) / np.float32(3.0)
+    assert np.float32(7.0) / np.float32(3.0) != np.float32(7.0) * (np.float32(1.0) / np.float32(3.0))
+    y = np.random.default_rng(5).uniform(-1, 1, (24, 64)).astype(np.float32)
+    assert np.array_equal(orc.rowmean_f32(y), orc.rowsum_f32(y) / np.float32(64))
+
+
 # ---- transpose ---------------------------------------------------------------------
 def test_transpose_golden(orc):
     g = GOLD["transpose_f32_10x20"]
