@@ -16,6 +16,9 @@
  *   relu, softmax, row-sum, transpose, gemm (f32 / f16 / bf16 inputs), bias add,
  *   half->float, bfloat->float, allclose, stats   : reference golden vectors
  *       and closed forms (tests/golden, tests/test_oracle.py);
+ *   row mean                                      : closed forms (the reference's test draws
+ *       random inputs and holds no vector): exact dyadic rows, sequential-order witnesses,
+ *       a true division;
  *   stats (reference median formula)              : also the reference's own
  *       ExecutionEngineUtils.cpp compiled into oracle/_ref;
  *   float->half / float->bfloat rounding          : exhaustive comparison with
