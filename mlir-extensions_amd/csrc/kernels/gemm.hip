@@ -249,9 +249,10 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
 
 // kAT / kBT as in gemm_scalar.  A is KContig unless transposed; B is KContig only
 // when transposed.
+// One 256 x 256 tile of C: tile number `id` of a tilesM x tilesN grid.
 template <typename T, bool kAT, bool kBT, typename Epi>
-__device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
-                                           int64_t M, int64_t N, int64_t K, Epi epi, char *lds) {
+__device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, int64_t M,
+                                          int64_t N, int64_t K, Epi epi, char *lds, int tilesM, int tilesN, int id) {
   static_assert(TI == 4 && TJ == 2 && kWaves == 8, "written for 8 wavefronts of 4 x 2 MFMA tiles");
   LdsChar *lds_base = (LdsChar *)lds;
   const int tid = threadIdx.x;
@@ -259,13 +260,8 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
   const int wave = tid >> 6;
   const int wm = wave / kWavesN, wn = wave % kWavesN;
 
-  // -- workgroup id -> tile, XCD-aware ------------------------------------------------
-  const int tilesM = int((M + BM - 1) / BM), tilesN = int((N + BN - 1) / BN);
+  // -- tile number -> tile, XCD-aware -------------------------------------------------
   const int tiles = tilesM * tilesN;
-  // Workgroups stride over the tiles: a launch with fewer workgroups than tiles still covers C, one
-  // with more leaves the surplus nothing to do.
-  const int workgroups = gridDim.x * gridDim.y;
-  for (int id = blockIdx.y * gridDim.x + blockIdx.x; id < tiles; id += workgroups) {
   int pid = id;
   if (tiles % 8 == 0)
     pid = (pid % 8) * (tiles / 8) + pid / 8; // ids congruent mod 8 share an XCD
@@ -373,9 +369,20 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
             epi(m, n, N, acc[i][j][r]);
         }
   }
-  if (id + workgroups < tiles)
-    __syncthreads(); // the ring is reused by this workgroup's next tile
-  } // tiles of this workgroup
+}
+
+// Workgroups stride over the tiles: a launch with fewer workgroups than tiles still covers C, one
+// with more leaves the surplus nothing to do.
+template <typename T, bool kAT, bool kBT, typename Epi>
+__device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
+                                           int64_t M, int64_t N, int64_t K, Epi epi, char *lds) {
+  const int tilesM = int((M + BM - 1) / BM), tilesN = int((N + BN - 1) / BN);
+  const int tiles = tilesM * tilesN, workgroups = gridDim.x * gridDim.y;
+  for (int id = blockIdx.y * gridDim.x + blockIdx.x; id < tiles; id += workgroups) {
+    gemm_tile<T, kAT, kBT, Epi>(A, B, M, N, K, epi, lds, tilesM, tilesN, id);
+    if (id + workgroups < tiles)
+      __syncthreads(); // the ring is reused by this workgroup's next tile
+  }
 }
 
 template <typename T, bool kAT, bool kBT, typename Epi>
