@@ -193,3 +193,17 @@ def test_driver_report_mode(tmp_path):
     assert timed[0].startswith("relu_f32_4096x4096: the kernel execution time is (ms, on HIP runtime):avg: ")
     assert timed[1].startswith("softmax_f16_16384x1024: the kernel execution time is (ms, on HIP runtime):avg: ")
     assert all(l.endswith("(over 5 runs)") for l in timed)
+
+
+def test_driver_runs_every_workload():
+    """Every workload the C++ driver lists goes through the whole ABI sequence once
+    (allocate, fill, copy, load, launch, time, copy back, free) and reports a rate."""
+    exe = os.path.join(REPO, "mlir-extensions_amd", "lib", "imex-hip-bench")
+    listed = subprocess.run([exe, "--list"], stdout=subprocess.PIPE, text=True, timeout=60).stdout.split("\n")
+    names = [l.split()[0] for l in listed if l.strip()]
+    assert len(names) >= 20
+    r = subprocess.run([exe, "--runs", "3", "--warmups", "1", "all"], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                       text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    for n in names:
+        assert any(l.startswith(n + ": back-to-back") for l in r.stdout.splitlines()), n
