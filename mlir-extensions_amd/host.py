@@ -179,9 +179,11 @@ def _pack_params(args):
 class Stream:
     """gpux stream: the object every gpu* call takes first (GPUToGPUX.cpp:36-59)."""
 
-    def __init__(self):
+    def __init__(self, hip_stream=None):
+        """`hip_stream`: an existing hipStream_t (integer handle) for the queue to run on instead of
+        creating its own; the queue does not destroy it."""
         self.rt = runtime()
-        self.handle = self.rt.gpuCreateStream(None, None)
+        self.handle = self.rt.gpuCreateStream(None, hip_stream)
         self._events = []
 
     def close(self):

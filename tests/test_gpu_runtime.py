@@ -207,3 +207,46 @@ def test_driver_runs_every_workload():
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     for n in names:
         assert any(l.startswith(n + ": back-to-back") for l in r.stdout.splitlines()), n
+
+
+def test_adopted_stream_and_graph_replay(host, orc):
+    """A queue built on a caller's hipStream_t (the `context` argument of gpuCreateStream) launches
+    on that stream, so a launch-bound sequence can be captured into a HIP graph and replayed:
+    here the fused chain out = (log a + |b|) - a feeding a ReLU, three replays with fresh inputs,
+    each checked against the oracle and against the same two launches run eagerly."""
+    import ctypes as C
+    import numpy as np
+    hip = C.CDLL("libamdhip64.so")
+    raw = C.c_void_p()
+    assert hip.hipStreamCreateWithFlags(C.byref(raw), 1) == 0  # non-blocking, default priority
+    s = host.Stream(hip_stream=raw.value)
+    n = 70000
+    a = orc.fill_uniform(n, "f32", 201, 0.5, 3.0)
+    b = orc.fill_uniform(n, "f32", 202, -3.0, 3.0)
+    d_a, d_b, d_t, d_o = s.to_device(a), s.to_device(b), s.alloc(n * 4), s.alloc(n * 4)
+    chain = s.prepare("imex_loop_fusion_f32", [n], [d_a, d_b, d_t, n])
+    relu = s.prepare("imex_relu_f32", [n], [d_t, d_o, n])
+    chain(), relu()   # eager once: modules loaded, kernels resolved, nothing left to allocate under capture
+    s.wait()
+    want = orc.relu_f32(orc.loop_fusion_f32(a, b))
+    assert np.array_equal(s.from_device(d_o, (n,), np.float32).view(np.uint32), want.view(np.uint32))
+
+    graph, exe = C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamBeginCapture(raw, 2) == 0          # relaxed mode
+    chain(), relu()
+    assert hip.hipStreamEndCapture(raw, C.byref(graph)) == 0
+    assert hip.hipGraphInstantiate(C.byref(exe), graph, None, None, C.c_size_t(0)) == 0
+    for seed in (203, 204, 205):
+        a2 = orc.fill_uniform(n, "f32", seed, 0.5, 3.0)
+        s.copy(d_a, a2.ctypes.data, n * 4)                  # new input, same buffers
+        s.copy(d_o, np.zeros(n, np.float32).ctypes.data, n * 4)
+        assert hip.hipGraphLaunch(exe, raw) == 0
+        s.wait()
+        got = s.from_device(d_o, (n,), np.float32)
+        assert np.array_equal(got.view(np.uint32), orc.relu_f32(orc.loop_fusion_f32(a2, b)).view(np.uint32)), seed
+    assert hip.hipGraphExecDestroy(exe) == 0 and hip.hipGraphDestroy(graph) == 0
+    for p in (d_a, d_b, d_t, d_o):
+        s.free(p)
+    s.close()                                               # must leave the adopted stream alive
+    assert hip.hipStreamSynchronize(raw) == 0
+    assert hip.hipStreamDestroy(raw) == 0
