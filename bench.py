@@ -39,6 +39,70 @@ def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
 
+# ---- seeded synthetic inputs -------------------------------------------------------------------
+# The raw output stream of std::mt19937 (numpy's MT19937 with the classic integer seeding is the
+# same generator) and the transforms of the benchmark definition: uniform u = (w >> 8) * 2^-24,
+# x = lo + (hi - lo) u in f64; normal by Box-Muller in f64 on two such uniforms; raw bit patterns
+# with NaN encodings redrawn.  f64 -> f32 -> f16 / bf16, each step round-to-nearest-even.
+def _mt19937_raw(seed, n):
+    bitgen = np.random.MT19937()
+    bitgen._legacy_seeding(seed)
+    return bitgen.random_raw(n).astype(np.uint32)
+
+
+def _narrow(x64, dtype):
+    f = x64.astype(np.float32)
+    if dtype == "f32":
+        return f
+    if dtype == "f16":
+        return f.astype(np.float16).view(np.uint16)
+    u = f.view(np.uint32)
+    rounded = ((u + (((u >> 16) & 1) + 0x7fff)) >> 16).astype(np.uint16)
+    nan = (u & 0x7fffffff) > 0x7f800000
+    return np.where(nan, np.where(u >> 31, 0xffc0, 0x7fc0).astype(np.uint16), rounded)
+
+
+def gen_uniform(n, dtype, seed, lo, hi):
+    u = (_mt19937_raw(seed, n) >> 8).astype(np.float64) * (1.0 / 16777216.0)
+    return _narrow(lo + (hi - lo) * u, dtype)
+
+
+def gen_normal(n, dtype, seed, mu, sigma):
+    pairs = (n + 1) // 2
+    w = _mt19937_raw(seed, 2 * pairs)
+    u1 = ((w[0::2] >> 8) + 1).astype(np.float64) * (1.0 / 16777216.0)
+    u2 = (w[1::2] >> 8).astype(np.float64) * (1.0 / 16777216.0)
+    r, angle = np.sqrt(-2.0 * np.log(u1)), 6.283185307179586476925286766559 * u2
+    out = np.empty(2 * pairs, np.float64)
+    out[0::2] = mu + sigma * (r * np.cos(angle))
+    out[1::2] = mu + sigma * (r * np.sin(angle))
+    return _narrow(out[:n], dtype)
+
+
+def gen_bits(n, dtype, seed):
+    """Raw words masked to the element width, NaN encodings skipped (each element takes the next
+    word of the stream that is not a NaN)."""
+    out = np.empty(0, np.uint32)
+    drawn = 0
+    stream = _mt19937_raw(seed, n + n // 16 + 1024)   # f16 words are NaNs 3 % of the time
+    while True:
+        w = stream[drawn:]
+        if dtype == "f32":
+            keep = ~(((w & 0x7f800000) == 0x7f800000) & ((w & 0x007fffff) != 0))
+            vals = w[keep]
+        else:
+            h = w & 0xffff
+            exp, man = (0x7c00, 0x03ff) if dtype == "f16" else (0x7f80, 0x007f)
+            vals = h[~(((h & exp) == exp) & ((h & man) != 0))]
+        out = np.concatenate([out, vals])
+        if out.size >= n:
+            break
+        drawn = stream.size
+        stream = _mt19937_raw(seed, 2 * stream.size)   # the same stream, longer
+    out = out[:n]
+    return out.view(np.float32) if dtype == "f32" else out.astype(np.uint16)
+
+
 class Workload:
     """One BASELINE.json configuration: device buffers, the kernel launch, its algorithmic
     work and the matching CPU-baseline call."""
@@ -74,8 +138,8 @@ def build_workloads(host, orc, stream, only):
         M = N = K = 4096
         cur = Workload("gemm_f16_4096", "imex_gemm_f16_f16_f32", [M, N, K], "mfma", 2.0 * M * N * K, "TFLOP/s",
                        "f16", "C[4096,4096] f32 = A[4096,4096] f16 . B[4096,4096] f16, uniform(-1,1), seeds 20246/20247")
-        a = orc.fill_uniform(M * K, "f16", 20246, -1.0, 1.0).reshape(M, K)
-        b = orc.fill_uniform(K * N, "f16", 20247, -1.0, 1.0).reshape(K, N)
+        a = gen_uniform(M * K, "f16", 20246, -1.0, 1.0).reshape(M, K)
+        b = gen_uniform(K * N, "f16", 20247, -1.0, 1.0).reshape(K, N)
         cur.args = [dev(a), dev(b), out(M * N * 4), M, N, K]
         rows = 4096
 
@@ -89,9 +153,9 @@ def build_workloads(host, orc, stream, only):
         M, K, N = 4096, 4096, 11008
         cur = Workload("gemm_mlp_bf16", "imex_gemm_bf16_bias_silu_bf16", [M, N, K], "mfma", 2.0 * M * N * K, "TFLOP/s",
                        "bf16", "out[4096,11008] bf16 = silu(A[4096,4096] bf16 . B[4096,11008] bf16 + bias f32), seeds 20248-20250")
-        a = orc.fill_normal(M * K, "bf16", 20248, 0.0, 1.0).reshape(M, K)
-        b = orc.fill_normal(K * N, "bf16", 20249, 0.0, 0.02).reshape(K, N)
-        bias = orc.fill_normal(N, "f32", 20250, 0.0, 0.1)
+        a = gen_normal(M * K, "bf16", 20248, 0.0, 1.0).reshape(M, K)
+        b = gen_normal(K * N, "bf16", 20249, 0.0, 0.02).reshape(K, N)
+        bias = gen_normal(N, "f32", 20250, 0.0, 0.1)
         cur.args = [dev(a), dev(b), dev(bias), out(M * N * 2), M, N, K]
         rows = 64
 
@@ -105,7 +169,7 @@ def build_workloads(host, orc, stream, only):
         n = 4096 * 4096
         cur = Workload("relu_f32", "imex_relu_f32", [n], "hbm", 2.0 * n * 4, "GB/s", "f32",
                        "relu f32 [4096,4096] uniform(-1,1) seed 20241, out of place")
-        x = orc.fill_uniform(n, "f32", 20241, -1.0, 1.0)
+        x = gen_uniform(n, "f32", 20241, -1.0, 1.0)
         cur.args = [dev(x), out(n * 4), n]
         cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_relu_f32(x, 2, 10) * 1e6), "full tensor, 2 warm-ups + 10 timed calls")
         wl.append(cur)
@@ -114,7 +178,7 @@ def build_workloads(host, orc, stream, only):
         rows, cols = 16384, 1024
         cur = Workload("softmax_f16", "imex_softmax_f16", [rows, cols], "hbm", 2.0 * rows * cols * 2, "GB/s", "f16",
                        "softmax f16 [16384,1024] normal(0,2) seed 20242, f32 internals")
-        x = orc.fill_normal(rows * cols, "f16", 20242, 0.0, 2.0).reshape(rows, cols)
+        x = gen_normal(rows * cols, "f16", 20242, 0.0, 2.0).reshape(rows, cols)
         cur.args = [dev(x), out(rows * cols * 2), rows, cols]
         cur.cpu = lambda x=x: (2.0 * x.size * 2 / (orc.time_softmax_f16(x, 1, 3) * 1e6), "full tensor, 1 warm-up + 3 timed calls")
         wl.append(cur)
@@ -123,7 +187,7 @@ def build_workloads(host, orc, stream, only):
         rows = cols = 8192
         cur = Workload("rowsum_f32", "imex_rowsum_f32", [rows, cols], "hbm", rows * cols * 4.0 + rows * 4.0, "GB/s",
                        "f32", "row-sum f32 [8192,8192] uniform(0,1) seed 20243 -> [8192]")
-        x = orc.fill_uniform(rows * cols, "f32", 20243, 0.0, 1.0).reshape(rows, cols)
+        x = gen_uniform(rows * cols, "f32", 20243, 0.0, 1.0).reshape(rows, cols)
         cur.args = [dev(x), out(rows * 4), rows, cols, 0.0]
         cur.cpu = lambda x=x: ((x.size * 4.0 + x.shape[0] * 4.0) / (orc.time_rowsum_f32(x, 1, 5) * 1e6), "full tensor, 1 warm-up + 5 timed calls")
         wl.append(cur)
@@ -132,7 +196,7 @@ def build_workloads(host, orc, stream, only):
         rows = cols = 8192
         cur = Workload("transpose_bf16", "imex_transpose2d_b16", [rows, cols], "hbm", 2.0 * rows * cols * 2, "GB/s",
                        "bf16", "transpose bf16 [8192,8192] random non-NaN bits seed 20244")
-        x = orc.fill_bits(rows * cols, "bf16", 20244).reshape(rows, cols)
+        x = gen_bits(rows * cols, "bf16", 20244).reshape(rows, cols)
         cur.args = [dev(x), out(rows * cols * 2), rows, cols]
         cur.cpu = lambda x=x: (2.0 * x.size * 2 / (orc.time_transpose2d(x, 1, 3) * 1e6), "full tensor, 1 warm-up + 3 timed calls")
         wl.append(cur)
@@ -141,7 +205,7 @@ def build_workloads(host, orc, stream, only):
         rows = cols = 4096
         cur = Workload("transpose_f32", "imex_transpose2d_b32", [rows, cols], "hbm", 2.0 * rows * cols * 4, "GB/s",
                        "f32", "transpose f32 [4096,4096] random non-NaN bits seed 20245")
-        x = orc.fill_bits(rows * cols, "f32", 20245).reshape(rows, cols)
+        x = gen_bits(rows * cols, "f32", 20245).reshape(rows, cols)
         cur.args = [dev(x), out(rows * cols * 4), rows, cols]
         cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_transpose2d(x, 1, 5) * 1e6), "full tensor, 1 warm-up + 5 timed calls")
         wl.append(cur)
@@ -150,7 +214,7 @@ def build_workloads(host, orc, stream, only):
         n = 512 * 640 * 20 * 15
         cur = Workload("silu_f32", "imex_silu_f32", [n], "hbm", 2.0 * n * 4, "GB/s", "f32",
                        "silu f32 512x640x20x15 uniform(-8,8) seed 20251")
-        x = orc.fill_uniform(n, "f32", 20251, -8.0, 8.0)
+        x = gen_uniform(n, "f32", 20251, -8.0, 8.0)
         cur.args = [dev(x), out(n * 4), n]
         cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_silu_f32(x, 0, 2) * 1e6), "full tensor, 2 timed calls")
         wl.append(cur)
@@ -299,7 +363,7 @@ def main():
 
     pkg = entry.load_package()
     host = pkg.host
-    orc = entry.load_oracle()
+    orc = None if args.no_cpu else entry.load_oracle()  # the oracle only ever runs as the CPU baseline
     host.runtime()
     host.kernels()  # raises if the HIP libraries are not built: there is no fallback
 
