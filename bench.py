@@ -321,7 +321,8 @@ def measure_reference_suite(stream):
             run("relu_%s_%s" % (dt, "x".join(map(str, shape))), "imex_relu_" + dt, [n], [n * w, n * w], [n])
     for shape in ((1, 1024, 40, 30), (50, 20, 3072), (512, 640, 20, 15)):
         n = int(np.prod(shape))
-        run("silu_f32_%s" % "x".join(map(str, shape)), "imex_silu_f32", [n], [n * 4, n * 4], [n])
+        for dt in ("f32", "f16"):
+            run("silu_%s_%s" % (dt, "x".join(map(str, shape))), "imex_silu_" + dt, [n], [n * width[dt]] * 2, [n])
     for rows in (1, 16, 64, 256, 1024):
         for dt, w in width.items():
             n = rows * 2000
@@ -335,7 +336,9 @@ def measure_reference_suite(stream):
             n = d[0] * d[1] * d[2] * bits // 8
             run("transpose_b%d_%dx%dx%d" % ((bits,) + d), "imex_transpose3d_b%d" % bits, list(d), [n, n], list(d))
     inner = 16 * 512 * 512
-    run("reduce_f32_32x16x512x512", "imex_reduce_outer_f32", [32, inner], [32 * inner * 4, inner * 4], [32, inner, 0.0])
+    for dt, w in width.items():
+        run("reduce_%s_32x16x512x512" % dt, "imex_reduce_outer_" + dt, [32, inner], [32 * inner * w, inner * w],
+            [32, inner, 0.0])
     for dt, w in width.items():
         n = 512 * 1024
         run("loop_fusion_%s_512x1024" % dt, "imex_loop_fusion_" + dt, [n], [n * w] * 3, [n])

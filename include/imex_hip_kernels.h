@@ -15,7 +15,7 @@
  * Kernels (name : arguments : reference op body it replaces)
  *   imex_relu_f32 / _f16 / _bf16   (in, out, n:i64)
  *       benchmarks/relu/relu_gpu.mlir.in:3-13            dims = {n}
- *   imex_silu_f32                  (in, out, n:i64)
+ *   imex_silu_f32 / _f16 / _bf16   (in, out, n:i64)
  *       benchmarks/silu/silu_gpu.mlir.in:3-19            dims = {n}
  *   imex_softmax_f32 / _f16 / _bf16 (in, out, rows:i64, cols:i64)
  *       benchmarks/softmax/softmax_gpu.mlir.in:4-44      dims = {rows, cols}
@@ -23,7 +23,7 @@
  *       WG/reduction_2D_1D_cross_sg_cross_lane.mlir:31-37 dims = {rows, cols}
  *   imex_rowmean_f32               (in, out, rows:i64, cols:i64)   out[r] = (sum_c in[r,c]) / cols
  *       WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir:51-52   dims = {rows, cols}
- *   imex_reduce_outer_f32          (in, out, outer:i64, inner:i64, init:f32)
+ *   imex_reduce_outer_f32 / _f16 / _bf16  (in, out, outer:i64, inner:i64, init:f32)
  *       benchmarks/reduce/reduce_gpu.mlir.in:4-21        dims = {outer, inner}
  *   imex_transpose2d_b16 / _b32    (in, out, rows:i64, cols:i64)
  *       benchmarks/transpose/transpose2d_gpu.mlir.in:4-11 dims = {rows, cols}

@@ -22,6 +22,10 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h16) {
   return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h16)));
 }
 __device__ __forceinline__ uint32_t float_to_half_bits(float f) {
+  // The empty asm keeps the conversion a conversion.  Left to itself the compiler folds a
+  // multiplication that feeds it into v_fma_mixlo_f16 a, b, 0 -- and (-0) + (+0) is +0, so a
+  // product that is exactly -0.0 (SiLU of a large negative input: 0 * x) would lose its sign.
+  asm volatile("" : "+v"(f));
   return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
 }
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t b16) { return u2f(b16 << 16); }
@@ -66,6 +70,50 @@ __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, __shfl_xor(v, off, kWave));
   return v;
 }
+
+// Element traits for kernels that exist in f32, f16 and bf16 forms: scalar get / put through
+// f32, and a 16-byte vector (u32x4) unpacked to / packed from kPerVec f32 values.  16-bit values
+// widen exactly and narrow with round-to-nearest-even.  (In a namespace of their own: kernels with
+// different needs keep local traits.)
+namespace io {
+enum class Dt { F32, F16, BF16 };
+template <Dt D> struct Elem;
+template <> struct Elem<Dt::F32> {
+  static constexpr int kBytes = 4, kPerVec = 4;
+  static __device__ __forceinline__ float get(const void *p, int64_t i) { return static_cast<const float *>(p)[i]; }
+  static __device__ __forceinline__ void put(void *p, int64_t i, float v) { static_cast<float *>(p)[i] = v; }
+  static __device__ __forceinline__ void unpack(u32x4 v, float *f) {
+    f[0] = u2f(v.x); f[1] = u2f(v.y); f[2] = u2f(v.z); f[3] = u2f(v.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float *f) { return u32x4{f2u(f[0]), f2u(f[1]), f2u(f[2]), f2u(f[3])}; }
+};
+template <bool kBf> struct Elem16 {
+  static constexpr int kBytes = 2, kPerVec = 8;
+  static __device__ __forceinline__ float widen(uint32_t h) { return kBf ? bf16_bits_to_float(h) : half_bits_to_float(h); }
+  static __device__ __forceinline__ uint32_t narrow(float f) { return kBf ? float_to_bf16_bits(f) : float_to_half_bits(f); }
+  static __device__ __forceinline__ float get(const void *p, int64_t i) { return widen(static_cast<const uint16_t *>(p)[i]); }
+  static __device__ __forceinline__ void put(void *p, int64_t i, float v) {
+    static_cast<uint16_t *>(p)[i] = static_cast<uint16_t>(narrow(v));
+  }
+  static __device__ __forceinline__ void unpack(u32x4 v, float *f) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = widen(w[i] & 0xffffu);
+      f[2 * i + 1] = widen(w[i] >> 16);
+    }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float *f) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      w[i] = narrow(f[2 * i]) | (narrow(f[2 * i + 1]) << 16);
+    return u32x4{w[0], w[1], w[2], w[3]};
+  }
+};
+template <> struct Elem<Dt::F16> : Elem16<false> {};
+template <> struct Elem<Dt::BF16> : Elem16<true> {};
+} // namespace io
 
 } // namespace imexhip
 #endif

@@ -158,6 +158,40 @@ struct SiluF32 {
   }
 };
 
+// 16-bit SiLU: widen to f32, the same five f32 operations, one rounding back to the 16-bit type
+// (the policy the reference applies to 16-bit element types on the GPU,
+// docs/Transforms/BF16ToGpu.md:17-26; benchmarks/silu/silu.dtypes.in lists f16).
+template <io::Dt D> struct Silu16 {
+  using E = io::Elem<D>;
+  SiluF32 f32;
+  __device__ __forceinline__ u32x4 vec(u32x4 v) const {
+    float f[E::kPerVec];
+    E::unpack(v, f);
+#pragma unroll
+    for (int i = 0; i < E::kPerVec; ++i)
+      f[i] = f32.one(f[i]);
+    return E::pack(f);
+  }
+  __device__ __forceinline__ void scalar(const void *in, void *out, int64_t i) const {
+    E::put(out, i, f32.one(E::get(in, i)));
+  }
+};
+
+// SiLU launch body: the 32-entry table staged in LDS (the index is data-dependent, and LDS serves
+// 64 different addresses per access where a constant load would not); below 4 Mi elements a lane's
+// exponentials and divisions are the critical path, so one vector per lane and pass instead of four.
+template <typename Op, int kElemBytes, typename Make>
+__device__ __forceinline__ void silu_launch(const void *in, void *out, int64_t n, Make make) {
+  __shared__ uint64_t table[32];
+  if (threadIdx.x < 32)
+    table[threadIdx.x] = kExp2Table[threadIdx.x];
+  __syncthreads();
+  if (n < (int64_t(1) << 22))
+    stream_map_impl<Op, kElemBytes, true, 1>(in, out, n, make(table));
+  else
+    stream_map<Op, kElemBytes>(in, out, n, make(table));
+}
+
 } // namespace
 
 extern "C" __global__ __launch_bounds__(kThreads) void imex_relu_f32(const float *in, float *out, int64_t n) {
@@ -175,16 +209,15 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_relu_bf16(const uint
 }
 
 extern "C" __global__ __launch_bounds__(kThreads) void imex_silu_f32(const float *in, float *out, int64_t n) {
-  // The 32-entry table is staged in LDS: the index is data-dependent, and LDS
-  // serves 64 different addresses per access where a constant load would not.
-  __shared__ uint64_t table[32];
-  if (threadIdx.x < 32)
-    table[threadIdx.x] = kExp2Table[threadIdx.x];
-  __syncthreads();
-  // Below 4 Mi elements a lane's exponentials and divisions are the critical path: one vector
-  // per lane and pass (four times the workgroups) instead of four.
-  if (n < (int64_t(1) << 22))
-    stream_map_impl<SiluF32, 4, true, 1>(in, out, n, SiluF32{table});
-  else
-    stream_map<SiluF32, 4>(in, out, n, SiluF32{table});
+  silu_launch<SiluF32, 4>(in, out, n, [](const uint64_t *table) { return SiluF32{table}; });
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_silu_f16(const uint16_t *in, uint16_t *out,
+                                                                    int64_t n) {
+  silu_launch<Silu16<io::Dt::F16>, 2>(in, out, n, [](const uint64_t *table) { return Silu16<io::Dt::F16>{SiluF32{table}}; });
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_silu_bf16(const uint16_t *in, uint16_t *out,
+                                                                     int64_t n) {
+  silu_launch<Silu16<io::Dt::BF16>, 2>(in, out, n, [](const uint64_t *table) { return Silu16<io::Dt::BF16>{SiluF32{table}}; });
 }

@@ -26,6 +26,7 @@
 #include "device_common.h"
 
 using namespace imexhip;
+using namespace imexhip::io;
 
 namespace {
 
@@ -102,43 +103,7 @@ __device__ __forceinline__ float input_chain(float a, float b, const LogfEntry *
   return t1 + t2;
 }
 
-enum class Dt { F32, F16, BF16 };
-template <Dt D> struct Elem;
-template <> struct Elem<Dt::F32> {
-  static constexpr int kBytes = 4, kPerVec = 4;
-  static __device__ __forceinline__ float get(const void *p, int64_t i) { return static_cast<const float *>(p)[i]; }
-  static __device__ __forceinline__ void put(void *p, int64_t i, float v) { static_cast<float *>(p)[i] = v; }
-  static __device__ __forceinline__ void unpack(u32x4 v, float *f) {
-    f[0] = u2f(v.x); f[1] = u2f(v.y); f[2] = u2f(v.z); f[3] = u2f(v.w);
-  }
-  static __device__ __forceinline__ u32x4 pack(const float *f) { return u32x4{f2u(f[0]), f2u(f[1]), f2u(f[2]), f2u(f[3])}; }
-};
-template <bool kBf> struct Elem16 {
-  static constexpr int kBytes = 2, kPerVec = 8;
-  static __device__ __forceinline__ float widen(uint32_t h) { return kBf ? bf16_bits_to_float(h) : half_bits_to_float(h); }
-  static __device__ __forceinline__ uint32_t narrow(float f) { return kBf ? float_to_bf16_bits(f) : float_to_half_bits(f); }
-  static __device__ __forceinline__ float get(const void *p, int64_t i) { return widen(static_cast<const uint16_t *>(p)[i]); }
-  static __device__ __forceinline__ void put(void *p, int64_t i, float v) {
-    static_cast<uint16_t *>(p)[i] = static_cast<uint16_t>(narrow(v));
-  }
-  static __device__ __forceinline__ void unpack(u32x4 v, float *f) {
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      f[2 * i] = widen(w[i] & 0xffffu);
-      f[2 * i + 1] = widen(w[i] >> 16);
-    }
-  }
-  static __device__ __forceinline__ u32x4 pack(const float *f) {
-    uint32_t w[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      w[i] = narrow(f[2 * i]) | (narrow(f[2 * i + 1]) << 16);
-    return u32x4{w[0], w[1], w[2], w[3]};
-  }
-};
-template <> struct Elem<Dt::F16> : Elem16<false> {};
-template <> struct Elem<Dt::BF16> : Elem16<true> {};
+// Elem<Dt>: element access, 16-byte vector unpack / pack to f32 (device_common.h).
 
 // ---- kLoopFusion: two streams in, one out ------------------------------------------
 // kVecs 16-byte vectors per lane and pass: four for tensors that stream from HBM, one for small

@@ -7,7 +7,7 @@
 //    (test/SPIRV/OpTest.Sum_FLOAT32.mlir:39); here a workgroup (or a wavefront,
 //    for short rows) owns a row, streams it once with 128-bit loads, and
 //    combines partial sums with wavefront-64 butterflies and one LDS hop.
-//  * imex_reduce_outer_f32: out[i] = init + sum_o in[o, i], the OUTERMOST
+//  * imex_reduce_outer_f32 / _f16 / _bf16: out[i] = init + sum_o in[o, i], the OUTERMOST
 //    dimension reduced (benchmarks/reduce/reduce_gpu.mlir.in:4-21).  Each lane
 //    owns groups of four adjacent outputs and adds the `outer` slices in order,
 //    which is the reference's summation order, so this one is bit-exact.
@@ -127,47 +127,87 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_rowmean_f32(const fl
 // spans per workgroup are what keeps the channels streaming (measured on 32 x 4 Mi: 111 us with
 // 4 KiB spans, 83 us with 32 KiB).  Loads of four slices are issued together, adds kept in slice
 // order.  Workgroups stride over the blocks of outputs, so any grid covers everything.
-template <int kVecs>
-__device__ __forceinline__ void reduce_outer_vec(const float *__restrict__ in, float *__restrict__ out, int64_t outer,
+template <io::Dt D, int kVecs>
+__device__ __forceinline__ void reduce_outer_vec(const void *__restrict__ in, void *__restrict__ out, int64_t outer,
                                                  int64_t inner, float init) {
-  constexpr int64_t kSpan = int64_t(kThreads) * 4 * kVecs; // outputs per workgroup and pass
-  const int64_t strideVecs = inner / 4;
+  using E = io::Elem<D>;
+  constexpr int kPer = E::kPerVec;                             // outputs per 16-byte vector: 4 or 8
+  constexpr int64_t kSpan = int64_t(kThreads) * kPer * kVecs;  // outputs per workgroup and pass
+  const u32x4 *src = static_cast<const u32x4 *>(in);
+  const int64_t strideVecs = inner / kPer;
   for (int64_t base = int64_t(blockIdx.x) * kSpan; base < inner; base += int64_t(gridDim.x) * kSpan) {
-    const int64_t i0 = base + threadIdx.x * 4;
-    f32x4 acc[kVecs];
+    const int64_t i0 = base + threadIdx.x * kPer;
+    float acc[kVecs][kPer];
 #pragma unroll
     for (int v = 0; v < kVecs; ++v)
-      acc[v] = f32x4{init, init, init, init};
-    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int e = 0; e < kPer; ++e)
+        acc[v][e] = init;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    auto add = [&](int v, u32x4 raw) {
+      float f[kPer];
+      E::unpack(raw, f);
+#pragma unroll
+      for (int e = 0; e < kPer; ++e)
+        acc[v][e] = acc[v][e] + f[e];
+    };
     int64_t o = 0;
     for (; o + 4 <= outer; o += 4) {
-      f32x4 t[4][kVecs];
+      u32x4 t[4][kVecs];
 #pragma unroll
       for (int u = 0; u < 4; ++u)
 #pragma unroll
         for (int v = 0; v < kVecs; ++v) {
-          const int64_t i = i0 + v * (kThreads * 4);
-          t[u][v] = i < inner ? __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(in + i) + (o + u) * strideVecs)
-                              : zero;
+          const int64_t i = i0 + v * (kThreads * kPer);
+          t[u][v] = i < inner ? __builtin_nontemporal_load(src + i / kPer + (o + u) * strideVecs) : zero;
         }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
 #pragma unroll
         for (int v = 0; v < kVecs; ++v)
-          acc[v] = acc[v] + t[u][v];
+          add(v, t[u][v]);
     }
     for (; o < outer; ++o)
 #pragma unroll
       for (int v = 0; v < kVecs; ++v) {
-        const int64_t i = i0 + v * (kThreads * 4);
+        const int64_t i = i0 + v * (kThreads * kPer);
         if (i < inner)
-          acc[v] = acc[v] + __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(in + i) + o * strideVecs);
+          add(v, __builtin_nontemporal_load(src + i / kPer + o * strideVecs));
       }
 #pragma unroll
     for (int v = 0; v < kVecs; ++v) {
-      const int64_t i = i0 + v * (kThreads * 4);
+      const int64_t i = i0 + v * (kThreads * kPer);
       if (i < inner)
-        *reinterpret_cast<f32x4 *>(out + i) = acc[v];
+        static_cast<u32x4 *>(out)[i / kPer] = E::pack(acc[v]);
+    }
+  }
+}
+
+// 16-bit inputs widen to f32, are added in f32 in slice order and rounded once at the end (the
+// reference's policy for 16-bit element types on the GPU, docs/Transforms/BF16ToGpu.md:17-26;
+// benchmarks/reduce/reduce.dtypes.in lists f32, f16, bf16).
+template <io::Dt D>
+__device__ __forceinline__ void reduce_outer(const void *in, void *out, int64_t outer, int64_t inner, float init) {
+  using E = io::Elem<D>;
+  const bool vec = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
+                   (inner % E::kPerVec) == 0;
+  if (vec) {
+    // the widest span that still leaves 512 workgroups (two per CU): 32, 16, 8 or 4 KiB per slice
+    const int64_t perVec = int64_t(kThreads) * E::kPerVec;
+    if (inner >= 512 * 8 * perVec)
+      reduce_outer_vec<D, 8>(in, out, outer, inner, init);
+    else if (inner >= 512 * 4 * perVec)
+      reduce_outer_vec<D, 4>(in, out, outer, inner, init);
+    else if (inner >= 512 * 2 * perVec)
+      reduce_outer_vec<D, 2>(in, out, outer, inner, init);
+    else
+      reduce_outer_vec<D, 1>(in, out, outer, inner, init);
+  } else {
+    for (int64_t i = int64_t(blockIdx.x) * kThreads + threadIdx.x; i < inner; i += int64_t(gridDim.x) * kThreads) {
+      float acc = init;
+      for (int64_t o = 0; o < outer; ++o)
+        acc = acc + E::get(in, o * inner + i);
+      E::put(out, i, acc);
     }
   }
 }
@@ -175,24 +215,17 @@ __device__ __forceinline__ void reduce_outer_vec(const float *__restrict__ in, f
 extern "C" __global__ __launch_bounds__(kThreads) void imex_reduce_outer_f32(const float *in, float *out,
                                                                             int64_t outer, int64_t inner,
                                                                             float init) {
-  const bool vec = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
-                   (inner % 4) == 0;
-  if (vec) {
-    // the widest span that still leaves 512 workgroups (two per CU): 32, 16, 8 or 4 KiB per slice
-    if (inner >= 512 * 8192)
-      reduce_outer_vec<8>(in, out, outer, inner, init);
-    else if (inner >= 512 * 4096)
-      reduce_outer_vec<4>(in, out, outer, inner, init);
-    else if (inner >= 512 * 2048)
-      reduce_outer_vec<2>(in, out, outer, inner, init);
-    else
-      reduce_outer_vec<1>(in, out, outer, inner, init);
-  } else {
-    for (int64_t i = int64_t(blockIdx.x) * kThreads + threadIdx.x; i < inner; i += int64_t(gridDim.x) * kThreads) {
-      float acc = init;
-      for (int64_t o = 0; o < outer; ++o)
-        acc = acc + in[o * inner + i];
-      out[i] = acc;
-    }
-  }
+  reduce_outer<io::Dt::F32>(in, out, outer, inner, init);
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_reduce_outer_f16(const uint16_t *in, uint16_t *out,
+                                                                            int64_t outer, int64_t inner,
+                                                                            float init) {
+  reduce_outer<io::Dt::F16>(in, out, outer, inner, init);
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_reduce_outer_bf16(const uint16_t *in, uint16_t *out,
+                                                                             int64_t outer, int64_t inner,
+                                                                             float init) {
+  reduce_outer<io::Dt::BF16>(in, out, outer, inner, init);
 }

@@ -28,7 +28,7 @@ extern const unsigned char imex_blob_probe[], imex_blob_probe_end[];
 namespace {
 
 enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm, Fusion, Attention, Probe };
-enum class Shape { Eltwise32, Eltwise16, Fusion32, Fusion16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, Attention, LanesOf512 };
+enum class Shape { Eltwise32, Eltwise16, Fusion32, Fusion16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, ReduceOuter16, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, Attention, LanesOf512 };
 
 struct Entry {
   const char *name;
@@ -43,6 +43,8 @@ const Entry kEntries[] = {
     {"imex_relu_f16", "(in: f16*, out: f16*, n: i64)", Module::Eltwise, Shape::Eltwise16, 1},
     {"imex_relu_bf16", "(in: bf16*, out: bf16*, n: i64)", Module::Eltwise, Shape::Eltwise16, 1},
     {"imex_silu_f32", "(in: f32*, out: f32*, n: i64)", Module::Eltwise, Shape::Fusion32, 1},
+    {"imex_silu_f16", "(in: f16*, out: f16*, n: i64)", Module::Eltwise, Shape::Fusion16, 1},
+    {"imex_silu_bf16", "(in: bf16*, out: bf16*, n: i64)", Module::Eltwise, Shape::Fusion16, 1},
     {"imex_softmax_f32", "(in: f32*, out: f32*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows32, 2},
     {"imex_softmax_f16", "(in: f16*, out: f16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows16, 2},
     {"imex_softmax_bf16", "(in: bf16*, out: bf16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows16, 2},
@@ -50,6 +52,10 @@ const Entry kEntries[] = {
     {"imex_rowmean_f32", "(in: f32*, out: f32*, rows: i64, cols: i64)", Module::Reduce, Shape::RowSum, 2},
     {"imex_reduce_outer_f32", "(in: f32*, out: f32*, outer: i64, inner: i64, init: f32)", Module::Reduce,
      Shape::ReduceOuter, 2},
+    {"imex_reduce_outer_f16", "(in: f16*, out: f16*, outer: i64, inner: i64, init: f32)", Module::Reduce,
+     Shape::ReduceOuter16, 2},
+    {"imex_reduce_outer_bf16", "(in: bf16*, out: bf16*, outer: i64, inner: i64, init: f32)", Module::Reduce,
+     Shape::ReduceOuter16, 2},
     {"imex_transpose2d_b32", "(in: b32*, out: b32*, rows: i64, cols: i64)", Module::Transpose, Shape::Transpose2D32, 2},
     {"imex_transpose2d_b16", "(in: b16*, out: b16*, rows: i64, cols: i64)", Module::Transpose, Shape::Transpose2D16, 2},
     {"imex_transpose3d_b32", "(in: b32*, out: b32*, d0: i64, d1: i64, d2: i64)", Module::Transpose,
@@ -176,10 +182,11 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
   case Shape::RowSum: // workgroup per row above 2048 columns, else wavefront per row
     grid[0] = dims[1] > 2048 ? static_cast<size_t>(dims[0]) : ceilDiv(dims[0], 4);
     break;
-  case Shape::ReduceOuter: { // 1024 v outputs per workgroup, v = 8, 4, 2, 1: the widest that leaves 512 workgroups
-    const int64_t inner = dims[1];
-    const int64_t v = inner >= 512 * 8192 ? 8 : inner >= 512 * 4096 ? 4 : inner >= 512 * 2048 ? 2 : 1;
-    grid[0] = ceilDiv(inner, 1024 * v);
+  case Shape::ReduceOuter:
+  case Shape::ReduceOuter16: { // 256 lanes x v vectors of 4 (8) outputs, v = 8, 4, 2, 1: the widest that leaves 512 workgroups
+    const int64_t inner = dims[1], perVec = e->shape == Shape::ReduceOuter ? 1024 : 2048;
+    const int64_t v = inner >= 512 * 8 * perVec ? 8 : inner >= 512 * 4 * perVec ? 4 : inner >= 512 * 2 * perVec ? 2 : 1;
+    grid[0] = ceilDiv(inner, perVec * v);
     break;
   }
   case Shape::Transpose2D32:

@@ -338,9 +338,9 @@ def relu(stream, x, dtype="f32"):
     return _unary(stream, "imex_relu_" + dtype, x, dtype, [x.size])
 
 
-def silu(stream, x):
-    """benchmarks/silu/silu_gpu.mlir.in:3-19"""
-    return _unary(stream, "imex_silu_f32", x, "f32", [x.size])
+def silu(stream, x, dtype="f32"):
+    """benchmarks/silu/silu_gpu.mlir.in:3-19 (f16 / bf16: bit patterns in, widened to f32, rounded once)"""
+    return _unary(stream, "imex_silu_" + dtype, x, dtype, [x.size])
 
 
 def _binary(stream, kernel, a, b, dtype, dims, out_shape):
@@ -430,11 +430,12 @@ def rowmean(stream, x):
     return _unary(stream, "imex_rowmean_f32", x, "f32", [rows, cols], out_shape=(rows,))
 
 
-def reduce_outer(stream, x, init=0.0):
-    """benchmarks/reduce/reduce_gpu.mlir.in:4-21: the outermost dim is summed away."""
+def reduce_outer(stream, x, init=0.0, dtype="f32"):
+    """benchmarks/reduce/reduce_gpu.mlir.in:4-21: the outermost dim is summed away (f16 / bf16: bit
+    patterns in and out, f32 accumulation)."""
     outer = x.shape[0]
     inner = int(np.prod(x.shape[1:]))
-    return _unary(stream, "imex_reduce_outer_f32", x, "f32", [outer, inner], extra=[float(init)],
+    return _unary(stream, "imex_reduce_outer_" + dtype, x, dtype, [outer, inner], extra=[float(init)],
                   out_shape=x.shape[1:])
 
 

@@ -242,6 +242,17 @@ void oracle_silu_f32(const float *x, float *y, size_t n) {
   for (size_t i = 0; i < n; ++i) y[i] = oracle_silu_scalar_f32(x[i]);
 }
 
+/* SiLU on 16-bit tensors: widen, the f32 chain above, one rounding (same policy;
+   benchmarks/silu/silu.dtypes.in lists f16). */
+void oracle_silu_16(const uint16_t *x, uint16_t *y, size_t n, int dtype) {
+  for (size_t i = 0; i < n; ++i) {
+    float in = dtype == ORACLE_F16 ? oracle_half_to_float(x[i]) : oracle_bfloat_to_float(x[i]);
+    float out;
+    oracle_silu_f32(&in, &out, 1);
+    y[i] = dtype == ORACLE_F16 ? oracle_float_to_half(out) : oracle_float_to_bfloat(out);
+  }
+}
+
 /* benchmarks/kLoopFusion/kLoopFusion.mlir.in:6-29: log, absf, addf, subf -- four
    separately rounded f32 ops; log is libm logf on the CPU path. */
 void oracle_loop_fusion_f32(const float *a, const float *b, float *out, size_t n) {
@@ -421,6 +432,20 @@ void oracle_reduce_outer_f32(const float *x, float *out, int64_t outer, int64_t 
     float acc = init;
     for (int64_t o = 0; o < outer; ++o) acc = acc + x[o * inner + i];
     out[i] = acc;
+  }
+}
+
+/* The same reduction on 16-bit tensors: every element widened to f32 (exact), added in f32 in the
+   same order, one rounding of the result (docs/Transforms/BF16ToGpu.md:17-26;
+   benchmarks/reduce/reduce.dtypes.in lists f16 and bf16). */
+void oracle_reduce_outer_16(const uint16_t *x, uint16_t *out, int64_t outer, int64_t inner, float init, int dtype) {
+  for (int64_t i = 0; i < inner; ++i) {
+    float acc = init;
+    for (int64_t o = 0; o < outer; ++o) {
+      uint16_t h = x[o * inner + i];
+      acc = acc + (dtype == ORACLE_F16 ? oracle_half_to_float(h) : oracle_bfloat_to_float(h));
+    }
+    out[i] = dtype == ORACLE_F16 ? oracle_float_to_half(acc) : oracle_float_to_bfloat(acc);
   }
 }
 

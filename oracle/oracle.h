@@ -70,6 +70,7 @@ void oracle_relu_f32(const float *x, float *y, size_t n);              /* benchm
 void oracle_relu_16(const uint16_t *x, uint16_t *y, size_t n, int dtype);
 void oracle_relu_olt_f32(const float *x, float *y, size_t n);          /* test/PlaidML/OpTest.Relu.mlir:29-35 */
 void oracle_silu_f32(const float *x, float *y, size_t n);              /* benchmarks/silu/silu_gpu.mlir.in:8-18 */
+void oracle_silu_16(const uint16_t *x, uint16_t *y, size_t n, int dtype);   /* widen, silu_f32, round once */
 float oracle_silu_scalar_f32(float x);
 void oracle_loop_fusion_f32(const float *a, const float *b, float *out, size_t n);                    /* benchmarks/kLoopFusion/kLoopFusion.mlir.in:6-29 */
 void oracle_input_fusion_f32(const float *a, const float *b, float *out, int64_t rows, int64_t cols); /* benchmarks/kInputFusion/kInputFusion.mlir.in:8-39 */
@@ -89,6 +90,7 @@ void oracle_softmax_16(const uint16_t *x, uint16_t *y, int64_t rows, int64_t col
 void oracle_rowsum_f32(const float *x, float *out, int64_t rows, int64_t cols, float init);       /* WG/reduction_2D_1D_cross_sg_cross_lane.mlir:31-37 */
 void oracle_rowmean_f32(const float *x, float *out, int64_t rows, int64_t cols);                      /* WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir:115-127 */
 void oracle_reduce_outer_f32(const float *x, float *out, int64_t outer, int64_t inner, float init); /* benchmarks/reduce/reduce_gpu.mlir.in:4-21 */
+void oracle_reduce_outer_16(const uint16_t *x, uint16_t *out, int64_t outer, int64_t inner, float init, int dtype); /* same, 16-bit in/out, f32 accumulation */
 float oracle_sum_all_f32(const float *x, int64_t n, float init);                                   /* test/PlaidML/OpTest.Sum.mlir:18-26 */
 
 /* ---- transpose ------------------------------------------------------------- */

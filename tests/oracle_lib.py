@@ -169,6 +169,13 @@ def silu_f32(x):
     return y
 
 
+def silu_16(x, dtype):
+    x = _c(x, np.uint16)
+    y = np.empty_like(x)
+    lib().oracle_silu_16(_p(x), _p(y), C.c_size_t(x.size), DT[dtype])
+    return y
+
+
 def loop_fusion_f32(a, b):
     a, b = _c(a, np.float32), _c(b, np.float32)
     out = np.empty_like(a)
@@ -220,6 +227,15 @@ def rowsum_f32(x, init=0.0):
     x = _c(x, np.float32)
     out = np.empty(x.shape[0], np.float32)
     lib().oracle_rowsum_f32(_p(x), _p(out), C.c_int64(x.shape[0]), C.c_int64(x.shape[1]), C.c_float(init))
+    return out
+
+
+def reduce_outer_16(x, dtype, init=0.0):
+    x = _c(x, np.uint16)
+    outer = x.shape[0]
+    inner = int(np.prod(x.shape[1:]))
+    out = np.empty(x.shape[1:], np.uint16)
+    lib().oracle_reduce_outer_16(_p(x), _p(out), C.c_int64(outer), C.c_int64(inner), C.c_float(init), DT[dtype])
     return out
 
 

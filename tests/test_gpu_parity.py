@@ -171,6 +171,29 @@ def test_rowsum_config_8192x8192(host, orc, stream):
     assert np.max(np.abs(got - exact) / exact) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_silu_sixteen_bit(host, orc, stream, dtype):
+    """benchmarks/silu/silu.dtypes.in lists f16: widen, the f32 chain, one rounding -- same bits as the oracle.
+    Every 16-bit pattern once (NaNs compared as NaNs), then the benchmark's 1x1024x40x30 and a large ragged size."""
+    every = np.arange(65536, dtype=np.uint16)
+    got, ref = host.silu(stream, every, dtype), orc.silu_16(every, dtype)
+    gf, rf = orc.to_float(got, dtype), orc.to_float(ref, dtype)
+    nan = np.isnan(rf)
+    assert np.array_equal(np.isnan(gf), nan) and np.array_equal(got[~nan], ref[~nan])
+    for n in (1024 * 40 * 30, (1 << 22) + 4099):
+        x = orc.fill_uniform(n, dtype, 304, -8.0, 8.0)
+        assert np.array_equal(host.silu(stream, x, dtype), orc.silu_16(x, dtype)), n
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", [(32, 16, 64, 64), (10, 24), (7, 1023), (3, 512 * 4096 + 16), (5, 512 * 2048 + 3)])
+def test_reduce_outer_sixteen_bit(host, orc, stream, dtype, shape):
+    """benchmarks/reduce/reduce.dtypes.in lists f16 and bf16: f32 accumulation in slice order, one rounding."""
+    x = orc.fill_uniform(int(np.prod(shape)), dtype, 305, -1.0, 1.0).reshape(shape)
+    got = host.reduce_outer(stream, x, init=0.25, dtype=dtype)
+    assert np.array_equal(got, orc.reduce_outer_16(x, dtype, init=0.25))
+
+
 def test_rowmean(host, orc, stream):
     """Mean over the last dimension (WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir: 1x24x1024x64,
     uniform(-1,1) inputs, checked there against the sequential CPU loop with allclose)."""

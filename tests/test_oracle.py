@@ -308,6 +308,21 @@ def test_rowsum_is_sequential(orc):
     assert orc.rowsum_f32(np.ones((1, 3), np.float32), init=2.5)[0] == 5.5
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_sixteen_bit_silu_and_outer_reduce_are_widen_compute_round(orc, dtype):
+    """The 16-bit forms are defined as: widen exactly, the f32 operation, one rounding.  Pinned by
+    composing the f32 oracle with the (exhaustively checked) conversions, and by exact cases."""
+    x = orc.fill_uniform(5000, dtype, 301, -8.0, 8.0)
+    assert np.array_equal(orc.silu_16(x, dtype), orc.from_float(orc.silu_f32(orc.to_float(x, dtype)), dtype))
+    assert orc.to_float(orc.silu_16(orc.from_float(np.zeros(3, np.float32), dtype), dtype), dtype).tolist() == [0, 0, 0]
+    m = orc.fill_int(7 * 300, dtype, 302, -8, 8).reshape(7, 300)
+    want = 0.5 + orc.to_float(m, dtype).sum(axis=0, dtype=np.float64)          # integers: exact in any order
+    assert np.array_equal(orc.to_float(orc.reduce_outer_16(m, dtype, init=0.5), dtype), want.astype(np.float32))
+    r = orc.fill_uniform(9 * 257, dtype, 303, -1.0, 1.0).reshape(9, 257)
+    assert np.array_equal(orc.reduce_outer_16(r, dtype, init=0.25),
+                          orc.from_float(orc.reduce_outer_f32(orc.to_float(r, dtype), init=0.25), dtype))
+
+
 def test_rowmean_closed_forms(orc):
     """WG/reduction_4D_3D_mean_intra_sg_intra_lane.mlir:115-127: sequential sum, then one division.
     Pinned by what arithmetic fixes: a constant dyadic row of a power-of-two length returns the constant
