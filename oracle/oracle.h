@@ -16,6 +16,8 @@
  *   relu, softmax, row-sum, transpose, gemm (f32 / f16 / bf16 inputs), bias add,
  *   half->float, bfloat->float, allclose, stats   : reference golden vectors
  *       and closed forms (tests/golden, tests/test_oracle.py);
+ *   silu / outer reduction on f16, bf16           : defined as widen -> f32 function -> one
+ *       rounding; pinned as that composition of the f32 oracle with the checked conversions;
  *   row mean                                      : closed forms (the reference's test draws
  *       random inputs and holds no vector): exact dyadic rows, sequential-order witnesses,
  *       a true division;
