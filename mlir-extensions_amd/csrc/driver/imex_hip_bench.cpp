@@ -87,6 +87,12 @@ std::vector<Workload> workloads() {
       {"gemm_f16_4096", "imex_gemm_f16_f16_f32", {K4, K4, K4},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true},
+      {"gemm_f16_4096_f16_out", "imex_gemm_f16_f16_f16", {K4, K4, K4},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true},
+      {"gemm_bf16_4096", "imex_gemm_bf16_bf16_f32", {K4, K4, K4},
+       {{Elem::BF16, {K4, K4}, true, -1, 1}, {Elem::BF16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true},
       {"gemm_f16_4096_transpose_b", "imex_gemm_f16_f16_f32_tb", {K4, K4, K4},
        {{Elem::F16, {K4, K4}, true, -0.5f, 0.5f}, {Elem::F16, {K4, K4}, true, -0.5f, 0.5f}, {Elem::F32, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true},
