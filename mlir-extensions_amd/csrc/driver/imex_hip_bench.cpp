@@ -146,9 +146,9 @@ std::vector<Workload> workloads() {
       // not operators: the MFMA pipe fed from LDS with nothing else going on, one workgroup per CU,
       // on hashed f16 operands in (-1,1) and on zeros -- the rate the GEMMs' operand values allow
       {"mfma_lds_ceiling_f16_random", "imex_mfma_lds_ceiling_f16", {256 * 512},
-       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 4096, 0}, 0, 256.0 * 8 * 4096 * 8 * 32768, true},
+       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 0}, 0, 256.0 * 8 * 2048 * 32 * 16384, true},
       {"mfma_lds_ceiling_f16_zeros", "imex_mfma_lds_ceiling_f16", {256 * 512},
-       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 4096, 1}, 0, 256.0 * 8 * 4096 * 8 * 32768, true},
+       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 1}, 0, 256.0 * 8 * 2048 * 32 * 16384, true},
   };
 }
 

@@ -13,8 +13,10 @@
 //
 // Blocking on MI355X:
 //   workgroup tile 256 x 256, 512 threads = 8 wavefronts in a 2 x 4 grid (two per
-//   SIMD), each owning 128 x 64 = 4 x 2 MFMA 32x32x16 tiles (128 accumulator
-//   registers);
+//   SIMD), each owning 128 x 64 = 8 x 4 MFMA 16x16x32 blocks (128 accumulator
+//   registers).  16x16x32 rather than 32x32x16: the two read the same LDS bytes per
+//   FLOP, but on random operands the part sustains about 9 % more with the former
+//   (the shader clock under MFMA load follows the operand values);
 //   K advances 32 at a time through a ring of four 32 KiB LDS stages: A and B
 //   tiles go from global memory STRAIGHT into LDS (buffer_load ... lds, 16 bytes
 //   per lane, no register staging) three steps ahead of the step that multiplies
@@ -26,10 +28,16 @@
 //   A fragments are 128-bit LDS reads; B is row-major [K,N] while the MFMA wants
 //   eight consecutive k per lane, so B fragments use the LDS transpose read
 //   (ds_read_b64_tr_b16) -- no permutes, no transposed copy of B anywhere;
-//   fragments are double-buffered in registers: the LDS reads of slice s+1 are
-//   placed by hand between the MFMAs of slice s (sched_barrier fences keep the
-//   order), and the barrier sits between a step's two slices so that eight
-//   MFMAs are always queued behind it;
+//   a K-step is multiplied in two halves of 16 MFMAs (the wavefront's upper, then
+//   lower four row blocks, each by all four column blocks); fragments are
+//   double-buffered in registers: the LDS reads the next half needs are placed by
+//   hand between the MFMAs of this one (sched_barrier fences keep the order), and
+//   the step's barrier sits between the halves so that sixteen MFMAs are always
+//   queued behind it;
+//   f32 results: the accumulator blocks of two neighbouring column blocks swap
+//   16-lane rows (v_permlane16_swap) so that every store instruction writes whole
+//   128-byte lines; 16-bit results: the product is taken transposed, which leaves
+//   four consecutive columns in a lane's registers -- one 8-byte store;
 //   workgroup ids are remapped so that the 32 workgroups resident on one XCD
 //   (ids congruent mod 8) cover a compact 4 x 8 block of tiles and share A and
 //   B panels in that XCD's L2.
@@ -58,7 +66,7 @@ constexpr int kThreads = 64 * kWaves;
 constexpr int BM = 256, BN = 256;
 constexpr int RK = 32;                              // K per step (one ring stage)
 constexpr int WM = BM / kWavesM, WN = BN / kWavesN; // wavefront tile
-constexpr int TI = WM / 32, TJ = WN / 32;           // MFMA 32x32 tiles per wavefront
+constexpr int FI = WM / 16, FJ = WN / 16;           // MFMA 16x16 tiles per wavefront: 8 x 4
 constexpr int kStages = 4;                          // LDS ring: 4 x 32 KiB of the 160 KiB
 constexpr int kImageBytes = 256 * RK * 2;           // one operand's 256 x 32 slab: 16 KiB
 constexpr int kRStage = 2 * kImageBytes;            // A image + B image
@@ -68,22 +76,24 @@ constexpr int kGroupM = 4;                          // tile rows per L2-sharing 
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));   // 4 floats at any float address
+typedef uint16_t u16x4u __attribute__((ext_vector_type(4), aligned(2))); // 4 halves at any half address
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) i16x4 LdsI16x4; // operand type of the LDS transpose read
 typedef __attribute__((address_space(3))) char LdsChar;
 
 struct F16 {
   using Frag = f16x8;
-  static __device__ __forceinline__ f32x16 mfma(Frag a, Frag b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  static __device__ __forceinline__ f32x4 mfma(Frag a, Frag b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ float widen(uint16_t h) { return half_bits_to_float(h); }
 };
 struct BF16 {
   using Frag = bf16x8;
-  static __device__ __forceinline__ f32x16 mfma(Frag a, Frag b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  static __device__ __forceinline__ f32x4 mfma(Frag a, Frag b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ float widen(uint16_t h) { return bf16_bits_to_float(h); }
 };
@@ -92,19 +102,27 @@ struct BF16 {
 #define IMEX_FENCE() __builtin_amdgcn_sched_barrier(0)
 
 // ---- epilogues ------------------------------------------------------------------
+// operator() takes one element of the accumulator.  kColumnsInRegisters picks how the tiled
+// path holds the accumulator: true = four consecutive columns of one row in a lane's four
+// registers, handed to vec4() (16-bit outputs: one 8-byte store per lane); false = one column
+// per lane, rows in the registers, stored element by element after the lane-row swap that
+// lines 32 consecutive columns up across lanes (32-bit outputs: whole 128-byte lines).
 struct StoreF32 {       // C = acc
+  static constexpr bool kColumnsInRegisters = false;
   float *C;
   __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
     __builtin_nontemporal_store(acc, C + m * N + n);
   }
 };
 struct AccumulateF32 {  // C = C + acc   (the reference kernel loads C as its initial accumulator)
+  static constexpr bool kColumnsInRegisters = false;
   float *C;
   __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
     C[m * N + n] = C[m * N + n] + acc;
   }
 };
 struct BiasAccumulateF32 { // C = bias[n] + (C + acc)  (bias.mlir:88-94,112-113)
+  static constexpr bool kColumnsInRegisters = false;
   float *C;
   const float *bias;
   __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
@@ -112,6 +130,7 @@ struct BiasAccumulateF32 { // C = bias[n] + (C + acc)  (bias.mlir:88-94,112-113)
   }
 };
 struct BiasSiluBF16 {   // out = bf16( silu( acc + bias[n] ) )
+  static constexpr bool kColumnsInRegisters = true;
   uint16_t *out;
   const float *bias;
   __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
@@ -119,11 +138,30 @@ struct BiasSiluBF16 {   // out = bf16( silu( acc + bias[n] ) )
     const float y = v / (1.0f + __expf(-v));
     out[m * N + n] = static_cast<uint16_t>(float_to_bf16_bits(y));
   }
+  __device__ __forceinline__ void vec4(int64_t m, int64_t n, int64_t N, f32x4 acc) const {
+    const f32x4 b = *reinterpret_cast<const f32x4u *>(bias + n);
+    u16x4u o;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float v = acc[r] + b[r];
+      const float y = v / (1.0f + __expf(-v));
+      o[r] = static_cast<uint16_t>(float_to_bf16_bits(y));
+    }
+    *reinterpret_cast<u16x4u *>(out + m * N + n) = o;
+  }
 };
 struct StoreF16 {       // C(f16) = acc   (WG/gemm_4kx4kx4k_f16_f16_f16.mlir)
+  static constexpr bool kColumnsInRegisters = true;
   uint16_t *C;
   __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
     C[m * N + n] = static_cast<uint16_t>(float_to_half_bits(acc));
+  }
+  __device__ __forceinline__ void vec4(int64_t m, int64_t n, int64_t N, f32x4 acc) const {
+    u16x4u o;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      o[r] = static_cast<uint16_t>(float_to_half_bits(acc[r]));
+    *reinterpret_cast<u16x4u *>(C + m * N + n) = o;
   }
 };
 
@@ -163,8 +201,8 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 }
 
 // One MFMA operand of a workgroup tile: a 256 x 32 (rows x k) slab per step.  Both
-// A (rows = m) and B (rows = n) want, per lane, row = lane % 32 of a 32-row
-// fragment and the 8 consecutive k starting at (lane / 32) * 8.
+// A (rows = m) and B (rows = n) want, per lane, row = lane % 16 of a 16-row
+// fragment and the 8 consecutive k starting at (lane / 16) * 8.
 //
 // KContig: the slab is k-contiguous in memory (A as [M,K], B as [N,K]).  LDS image
 //   [256 rows][32 k], 64-byte rows; 16-byte group c of row r is stored at group
@@ -183,7 +221,7 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
   int voff[kDmaPerWave];         // per-lane byte offset of each copy at step 0
   int step;                      // bytes per K-step in memory
   int dstWave;                   // LDS byte offset of this wavefront's copies inside the image
-  int rd[kStrided ? kFrags : 2]; // per-lane LDS read bases: KStrided one per fragment, KContig one per slice
+  int rd[kStrided ? kFrags : 1]; // per-lane LDS read bases: KStrided one per fragment, KContig one (fragments 1 KiB apart)
 
   // ptr: the operand's matrix; ld: its leading dimension; first: first row (m0 or n0)
   // of the slab; w0: the wavefront's first row inside the slab; extent: rows * cols.
@@ -204,10 +242,8 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
       }
       step = RK * 2;
       dstWave = wave * (256 / kWaves) * (RK * 2);
-      const int fragRow = lane & 31, fragHalf = lane >> 5;
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
-        rd[ks] = (w0 + fragRow) * (RK * 2) + ((((ks * 2 + fragHalf) ^ (fragRow >> 2)) & 3) << 4);
+      const int fragRow = lane & 15, kGroup = lane >> 4;
+      rd[0] = (w0 + fragRow) * (RK * 2) + (((kGroup ^ (fragRow >> 2)) & 3) << 4);
     } else {
       rsrc = make_rsrc(ptr + first, (extent - first) * 2);
 #pragma unroll
@@ -220,12 +256,12 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
       }
       step = int(RK * ld * 2);
       dstWave = wave * (RK / kWaves) * 512;
-      const int t = lane & 15, block = (lane >> 4) & 1, khalf = lane >> 5;
-      const int g = (t >> 2) | (khalf << 2); // g(k-row) for k-row = ks*16 + khalf*8 + h*4 + t/4
-      const int pair0 = w0 / 16 + block;     // 32-byte pair holding this lane's rows, fragment 0
+      const int t = lane & 15, kGroup = lane >> 4;
+      const int g = (t >> 2) | ((kGroup & 1) << 2); // g(k-row) for k-row = kGroup*8 + h*4 + t/4
+      const int pair0 = w0 / 16;                    // 32-byte pair holding fragment 0's rows
 #pragma unroll
       for (int f = 0; f < kFrags; ++f)
-        rd[f] = (khalf * 8 + (t >> 2)) * 512 + (((pair0 + 2 * f) ^ g) * 32) + (t & 3) * 8;
+        rd[f] = (kGroup * 8 + (t >> 2)) * 512 + (((pair0 + f) ^ g) * 32) + (t & 3) * 8;
     }
   }
   // the wavefront's copies of K-step kt into the image at LDS byte offset `image`
@@ -234,12 +270,12 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
     for (int q = 0; q < kDmaPerWave; ++q)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + image + dstWave + q * 1024, 16, voff[q], kt * step, 0, 0);
   }
-  // fragment f (rows w0 + 32 f ...) of 16-wide slice ks of the image at `image`
-  __device__ __forceinline__ typename T::Frag read(const char *lds, int image, int ks, int f) const {
+  // fragment f (rows w0 + 16 f ..., all 32 k) of the image at `image`
+  __device__ __forceinline__ typename T::Frag read(const char *lds, int image, int f) const {
     if constexpr (!kStrided) {
-      return *reinterpret_cast<const typename T::Frag *>(lds + image + rd[ks] + f * 32 * (RK * 2));
+      return *reinterpret_cast<const typename T::Frag *>(lds + image + rd[0] + f * 16 * (RK * 2));
     } else {
-      const char *p = lds + image + rd[f] + ks * 16 * 512;
+      const char *p = lds + image + rd[f];
       const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p));           // k +0..3
       const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p + 4 * 512)); // k +4..7
       return __builtin_bit_cast(typename T::Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
@@ -253,7 +289,7 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
 template <typename T, bool kAT, bool kBT, typename Epi>
 __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, int64_t M,
                                           int64_t N, int64_t K, Epi epi, char *lds, int tilesM, int tilesN, int id) {
-  static_assert(TI == 4 && TJ == 2 && kWaves == 8, "written for 8 wavefronts of 4 x 2 MFMA tiles");
+  static_assert(FI == 8 && FJ == 4 && kWaves == 8, "written for 8 wavefronts of 8 x 4 MFMA tiles");
   LdsChar *lds_base = (LdsChar *)lds;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -273,8 +309,8 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   const int64_t m0 = int64_t(tileM) * BM, n0 = int64_t(tileN) * BN;
 
   const int waveU = __builtin_amdgcn_readfirstlane(wave);
-  Operand<T, kAT, TI> opA;
-  Operand<T, !kBT, TJ> opB;
+  Operand<T, kAT, FI> opA;
+  Operand<T, !kBT, FJ> opB;
   opA.setup(A, kAT ? M : K, m0, wm * WM, M * K, waveU, lane);
   opB.setup(B, kBT ? K : N, n0, wn * WN, K * N, waveU, lane);
   constexpr int kImgA = 0, kImgB = kImageBytes;
@@ -283,30 +319,51 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
     opB.dma(lds_base, stageOff + kImgB, kt);
   };
 
-  f32x16 acc[TI][TJ];
+  // acc[i][j] is the 16 x 16 block at rows 16 i, columns 16 j of the wavefront's tile, held
+  // TRANSPOSED (the MFMA is given the B fragment as its first operand): lane l has row
+  // l % 16 and the four consecutive columns (l / 16) * 4 ..., which is one 16-byte store.
+  f32x4 acc[FI][FJ];
 #pragma unroll
-  for (int i = 0; i < TI; ++i)
+  for (int i = 0; i < FI; ++i)
 #pragma unroll
-    for (int j = 0; j < TJ; ++j)
+    for (int j = 0; j < FJ; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
+      for (int r = 0; r < 4; ++r)
         acc[i][j][r] = 0.0f;
 
-  typename T::Frag af[2][TI], bf[2][TJ];
-  auto read_a = [&](int stageOff, int ks, int buf, int i) { af[buf][i] = opA.read(lds, stageOff + kImgA, ks, i); };
-  auto read_b = [&](int stageOff, int ks, int buf, int j) { bf[buf][j] = opB.read(lds, stageOff + kImgB, ks, j); };
-  auto mm = [&](int buf, int i, int j) { acc[i][j] = T::mfma(af[buf][i], bf[buf][j], acc[i][j]); };
-  // 8 MFMAs from register buffer `buf`, interleaved by hand with the LDS reads that
-  // fill buf^1 (the fences keep the compiler from regrouping them)
-  auto slice = [&](int buf, int rOff, int rks) {
-    mm(buf, 0, 0); read_a(rOff, rks, buf ^ 1, 0); IMEX_FENCE();
-    mm(buf, 0, 1); read_a(rOff, rks, buf ^ 1, 1); IMEX_FENCE();
-    mm(buf, 1, 0); read_b(rOff, rks, buf ^ 1, 0); IMEX_FENCE();
-    mm(buf, 1, 1); read_a(rOff, rks, buf ^ 1, 2); IMEX_FENCE();
-    mm(buf, 2, 0); read_a(rOff, rks, buf ^ 1, 3); IMEX_FENCE();
-    mm(buf, 2, 1); read_b(rOff, rks, buf ^ 1, 1); IMEX_FENCE();
-    mm(buf, 3, 0); IMEX_FENCE();
-    mm(buf, 3, 1); IMEX_FENCE();
+  // A step multiplies the wavefront's upper four row fragments (half 0), then the lower four
+  // (half 1), each by all four B fragments.  af[h] holds half h's A fragments; bf[p] the B
+  // fragments of a step of parity p.
+  typename T::Frag af[2][FI / 2], bf[2][FJ];
+  auto read_a = [&](int stageOff, int h, int ii) { af[h][ii] = opA.read(lds, stageOff + kImgA, h * (FI / 2) + ii); };
+  auto read_b = [&](int stageOff, int p, int j) { bf[p][j] = opB.read(lds, stageOff + kImgB, j); };
+  auto mm = [&](int h, int p, int ii, int j) {
+    if constexpr (Epi::kColumnsInRegisters)
+      acc[h * (FI / 2) + ii][j] = T::mfma(bf[p][j], af[h][ii], acc[h * (FI / 2) + ii][j]);
+    else
+      acc[h * (FI / 2) + ii][j] = T::mfma(af[h][ii], bf[p][j], acc[h * (FI / 2) + ii][j]);
+  };
+  // half 0 of a step of parity p: 16 MFMAs, and between them the reads of this step's lower
+  // A fragments (the fences keep the compiler from regrouping them)
+  auto half0 = [&](int p, int curOff) {
+#pragma unroll
+    for (int ii = 0; ii < FI / 2; ++ii) {
+      mm(0, p, ii, 0); read_a(curOff, 1, ii); IMEX_FENCE();
+      mm(0, p, ii, 1); IMEX_FENCE();
+      mm(0, p, ii, 2); IMEX_FENCE();
+      mm(0, p, ii, 3); IMEX_FENCE();
+    }
+  };
+  // half 1: 16 MFMAs, and between them the reads of the NEXT step's upper A fragments and
+  // of its B fragments (into the other parity's registers)
+  auto half1 = [&](int p, int nxtOff) {
+#pragma unroll
+    for (int ii = 0; ii < FI / 2; ++ii) {
+      mm(1, p, ii, 0); read_a(nxtOff, 0, ii); IMEX_FENCE();
+      mm(1, p, ii, 1); IMEX_FENCE();
+      mm(1, p, ii, 2); read_b(nxtOff, p ^ 1, ii); IMEX_FENCE();
+      mm(1, p, ii, 3); IMEX_FENCE();
+    }
   };
 
   const int kTiles = int(K / RK);
@@ -319,55 +376,104 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   __builtin_amdgcn_s_barrier();
   IMEX_FENCE();
 #pragma unroll
-  for (int i = 0; i < TI; ++i) read_a(0, 0, 0, i);
+  for (int ii = 0; ii < FI / 2; ++ii) read_a(0, 0, ii);
 #pragma unroll
-  for (int j = 0; j < TJ; ++j) read_b(0, 0, 0, j);
+  for (int j = 0; j < FJ; ++j) read_b(0, 0, j);
   IMEX_FENCE();
 
   int curOff = 0;               // stage of tile t
   int nxtOff = kRStage;         // stage of tile t+1
   int dmaOff = kDist * kRStage; // stage tile t+kDist goes to (= stage of tile t-1)
-  for (int t = 0; t < kTiles; ++t) {
+  auto step = [&](int p, int t) {
     // The stage of tile t-1 is free: every wavefront passed the previous step's
     // barrier after its last reads of it.  Past the end of K the copies re-fetch the
     // last tile into a stage nobody reads, so every step is the same code.
     dma_tile(min(t + kDist, lastTile), dmaOff);
     IMEX_FENCE();
-    slice(0, curOff, 1);                            // multiplies k 0-15 of tile t, reads its k 16-31
+    half0(p, curOff);                               // rows 0-63 of tile t; reads its rows 64-127
     wait_vmcnt<(kDist - 1) * 2 * kDmaPerWave>();    // tile t+1 has landed (this wavefront's part) ...
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();                   // ... and everyone else's; all reads of tile t are done
     IMEX_FENCE();
-    slice(1, nxtOff, 0);                            // multiplies k 16-31 of tile t, reads k 0-15 of tile t+1
+    half1(p, nxtOff);                               // rows 64-127 of tile t; reads tile t+1's rows 0-63 and B
     curOff = nxtOff;
     nxtOff = nxtOff + kRStage == kStages * kRStage ? 0 : nxtOff + kRStage;
     dmaOff = dmaOff + kRStage == kStages * kRStage ? 0 : dmaOff + kRStage;
+  };
+  int t = 0;
+  for (; t + 1 < kTiles; t += 2) { // two steps per trip, so that the B registers' parity is a literal
+    step(0, t);
+    step(1, t + 1);
   }
+  if (t < kTiles)
+    step(0, t);
   wait_vmcnt<0>();
 
-  // -- epilogue: lane holds, for tile (i,j), column n = lane%32 and rows
-  //    (r/4)*8 + (lane/32)*4 + r%4, r = 0..15.
-  const int fragRow = lane & 31, fragHalf = lane >> 5;
-  const int64_t mBase = m0 + wm * WM + fragHalf * 4, nBase = n0 + wn * WN + fragRow;
-  if (m0 + BM <= M && n0 + BN <= N) { // interior tile (uniform over the workgroup): nothing to mask
+  // -- epilogue.  kColumnsInRegisters: lane holds, for block (i,j), row lane%16 and columns
+  //    (lane/16)*4 + 0..3; otherwise column lane%16 and rows (lane/16)*4 + 0..3.
+  const bool interior = m0 + BM <= M && n0 + BN <= N; // uniform over the workgroup: nothing to mask
+  if constexpr (Epi::kColumnsInRegisters) {
+    const int64_t mBase = m0 + wm * WM + (lane & 15), nBase = n0 + wn * WN + (lane >> 4) * 4;
+    if (interior) {
 #pragma unroll
-    for (int i = 0; i < TI; ++i)
+      for (int i = 0; i < FI; ++i)
 #pragma unroll
-      for (int j = 0; j < TJ; ++j)
+        for (int j = 0; j < FJ; ++j)
+          epi.vec4(mBase + i * 16, nBase + j * 16, N, acc[i][j]);
+    } else {
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          epi(mBase + i * 32 + (r >> 2) * 8 + (r & 3), nBase + j * 32, N, acc[i][j][r]);
+      for (int i = 0; i < FI; ++i)
+#pragma unroll
+        for (int j = 0; j < FJ; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int64_t m = mBase + i * 16, n = nBase + j * 16 + r;
+            if (m < M && n < N)
+              epi(m, n, N, acc[i][j][r]);
+          }
+    }
   } else {
+    // Blocks j and j+1 sit side by side in C.  Swapping the odd 16-lane rows of one with the
+    // even rows of the other leaves lanes 0-31 of a register with 32 consecutive columns of
+    // one row of C and lanes 32-63 with the row 8 below: whole 128-byte lines per store.
+    const int64_t mBase = m0 + wm * WM + (lane >> 5) * 8, nBase = n0 + wn * WN + (lane & 31);
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); // the last MFMA results are in their registers
 #pragma unroll
-    for (int i = 0; i < TI; ++i)
+    for (int i = 0; i < FI; ++i)
 #pragma unroll
-      for (int j = 0; j < TJ; ++j)
+      for (int j = 0; j < FJ; j += 2)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int64_t m = mBase + i * 32 + (r >> 2) * 8 + (r & 3), n = nBase + j * 32;
-          if (m < M && n < N)
-            epi(m, n, N, acc[i][j][r]);
+        for (int r = 0; r < 4; ++r) {
+          // (written as an instruction: the compiler's own handling of the corresponding builtin
+          // lost track of the second result here; the waits on either side stand in for the
+          // hazard padding the compiler would add)
+          asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1"
+                       : "+v"(acc[i][j][r]), "+v"(acc[i][j + 1][r])); // -> rows r, r+8 | rows r+4, r+12
         }
+    if (interior) {
+#pragma unroll
+      for (int i = 0; i < FI; ++i)
+#pragma unroll
+        for (int j = 0; j < FJ; j += 2)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            epi(mBase + i * 16 + r, nBase + j * 16, N, acc[i][j][r]);
+            epi(mBase + i * 16 + r + 4, nBase + j * 16, N, acc[i][j + 1][r]);
+          }
+    } else {
+#pragma unroll
+      for (int i = 0; i < FI; ++i)
+#pragma unroll
+        for (int j = 0; j < FJ; j += 2)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int64_t m = mBase + i * 16 + r + 4 * h, n = nBase + j * 16;
+              if (m < M && n < N)
+                epi(m, n, N, acc[i][j + h][r]);
+            }
+    }
   }
 }
 

@@ -827,14 +827,14 @@ def _ceiling_lds_f16(workgroup):
 
 def test_mfma_ceiling_kernel_computes_what_it_says(host, stream):
     """No oracle and no reference counterpart: the expected sums follow from the published
-    operand / accumulator lane layout of MFMA 32x32x16 (A[m = l%32][k = 8(l/32)..+8],
-    B likewise in n, C[8(r/4) + 4(l/32) + r%4][l%32] in register r), in f64."""
+    operand / accumulator lane layout of MFMA 16x16x32 (A[m = l%16][k = 8(l/16)..+8],
+    B likewise in n, C[4(l/16) + r][l%16] in register r), in f64."""
     iters, groups = 5, 3
     say("mfma ceiling probe: %d workgroups x %d steps" % (groups, iters))
     got = host.mfma_lds_ceiling(stream, groups, iters)
     assert got.shape == (groups, 512)
     l = np.arange(64)
-    rows = (8 * (np.arange(16)[None, :] // 4) + 4 * (l[:, None] // 32) + np.arange(16)[None, :] % 4)  # [lane, r]
+    rows = 4 * (l[:, None] // 16) + np.arange(4)[None, :]                      # [lane, r]
     for g in range(groups):
         slots = _ceiling_lds_f16(g)
         for w in range(8):
@@ -843,17 +843,17 @@ def test_mfma_ceiling_kernel_computes_what_it_says(host, stream):
             for it in range(iters):
                 off = (it & 63) * 64
                 frag = lambda base: slots[(lane + off + base) & 4095]          # [64 lanes, 8 k]
-                def tile(f):                                                     # -> [32, 16]
-                    t = np.zeros((32, 16))
-                    for k8 in range(2):
-                        t[:, 8 * k8:8 * k8 + 8] = f[32 * k8:32 * k8 + 32]
+                def tile(f):                                                     # -> [16, 32]
+                    t = np.zeros((16, 32))
+                    for k8 in range(4):
+                        t[:, 8 * k8:8 * k8 + 8] = f[16 * k8:16 * k8 + 16]
                     return t
-                for i in range(4):
-                    A = tile(frag(i * 512))
-                    for j in range(2):
-                        Bt = tile(frag(2048 + j * 512))                          # [n, k]
+                for i in range(8):
+                    A = tile(frag(i * 256))
+                    for j in range(4):
+                        Bt = tile(frag(2048 + j * 256))                          # [n, k]
                         Cm = A @ Bt.T
-                        total += Cm[rows, (l % 32)[:, None]].sum(axis=1)
+                        total += Cm[rows, (l % 16)[:, None]].sum(axis=1)
             want = total
             have = got[g, w * 64:(w + 1) * 64].astype(np.float64)
             assert np.all(np.abs(have - want) <= 1e-4 * np.abs(want).max() + 1e-4), (g, w)
