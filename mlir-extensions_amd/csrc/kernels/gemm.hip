@@ -206,8 +206,11 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 //
 // KContig: the slab is k-contiguous in memory (A as [M,K], B as [N,K]).  LDS image
 //   [256 rows][32 k], 64-byte rows; 16-byte group c of row r is stored at group
-//   c ^ ((r >> 2) & 3), which makes the 128-bit fragment reads conflict-free.  One
-//   1 KiB copy = 16 rows.  A fragment is one ds_read_b128.
+//   c ^ h((r >> 2) & 3), h = {0, 2, 3, 1}.  A fragment is one ds_read_b128 (lane: row
+//   lane % 16, group lane / 16); the LDS serves such a read 16 lanes at a time, and the
+//   lanes that go together are not neighbours (0-3 with 12-15, 20-23 and 24-27; 4-7 with
+//   8-11, 16-19 and 28-31; likewise in the upper half) -- h is chosen so that each of
+//   those sets touches every bank once.  One 1 KiB copy = 16 rows.
 // KStrided: the slab's rows are strided in memory (B as [K,N], A as [K,M]).  LDS
 //   image [32 k][256 rows], 512-byte rows; 32-byte pair p of k-row r at pair
 //   p ^ g(r), g(r) = (r & 3) | ((r >> 3 & 1) << 2).  One copy = 2 k-rows.  A
@@ -216,6 +219,8 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 //   receives 4 consecutive k of row t.
 // A direct global->LDS copy puts lane l's 16 bytes at base + 16 l, so the swizzle
 // is applied to the lane's GLOBAL address instead.
+__device__ __forceinline__ int kcontig_swizzle(int row) { return (0x78 >> (((row >> 2) & 3) * 2)) & 3; }
+
 template <typename T, bool kStrided, int kFrags> struct Operand {
   __amdgpu_buffer_rsrc_t rsrc;
   int voff[kDmaPerWave];         // per-lane byte offset of each copy at step 0
@@ -237,13 +242,13 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
 #pragma unroll
       for (int q = 0; q < kDmaPerWave; ++q) {
         const int row = wave * (256 / kWaves) + q * 16 + (lane >> 2);
-        const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+        const int chunk = (lane & 3) ^ kcontig_swizzle(row);
         voff[q] = int((int64_t(min(row, last)) * ld + chunk * 8) * 2);
       }
       step = RK * 2;
       dstWave = wave * (256 / kWaves) * (RK * 2);
       const int fragRow = lane & 15, kGroup = lane >> 4;
-      rd[0] = (w0 + fragRow) * (RK * 2) + (((kGroup ^ (fragRow >> 2)) & 3) << 4);
+      rd[0] = (w0 + fragRow) * (RK * 2) + ((kGroup ^ kcontig_swizzle(fragRow)) << 4);
     } else {
       rsrc = make_rsrc(ptr + first, (extent - first) * 2);
 #pragma unroll
