@@ -255,7 +255,7 @@ def measure_secondary(stream, w, rounds):
     IMEX-profiler protocol with a cache flush before each timed launch."""
     # MFMA-bound kernels get a long warm-up: coming from lighter work the part needs
     # ~100 launches before its clock settles under the new load
-    warm = 150 if w.bound == "mfma" else 3
+    warm = 150 if w.bound == "mfma" else 20
     hot_total = stream.profile(w.kernel, w.dims, w.args, warmups=warm, rounds=rounds, mode=1)[0]
     hot_ms = hot_total / rounds
     cold = stream.profile(w.kernel, w.dims, w.args, warmups=2, rounds=min(rounds, 20), flush_bytes=FLUSH_BYTES, mode=0)
@@ -395,7 +395,7 @@ def main():
     per = []
     secondary = sorted(workloads[1:], key=lambda w: w.bound == "mfma")  # the other GEMM goes last
     for w in secondary:
-        hot_ms, cold_ms = measure_secondary(stream, w, rounds=50)
+        hot_ms, cold_ms = measure_secondary(stream, w, rounds=50 if w.bound == "mfma" else 200)
         rot_ms, copies = measure_rotating(host, stream, w, passes=max(2, 200 // 24))
         rf = roofline(w, hot_ms)
         entry_ = {"name": w.name, "workload": w.describe, "kernel": w.kernel, "dtype": w.dtype,
