@@ -110,7 +110,8 @@ __device__ const uint64_t kExp2Table[32] = {
     0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
     0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
 
-__device__ __forceinline__ float expf_libm(float x, const uint64_t *table) {
+// The arithmetic of expf for an x libm sends down its main path (|x| < 88, finite).
+__device__ __forceinline__ float expf_libm_core(float x, const uint64_t *table) {
   constexpr double kInvLn2N = 0x1.71547652b82fep+0 * 32;
   constexpr double kShift = 0x1.8p+52;
   constexpr double kC0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32;
@@ -130,7 +131,11 @@ __device__ __forceinline__ float expf_libm(float x, const uint64_t *table) {
   double y = kC2 * r + 1.0;
   y = p * r2 + y;
   y = y * s;
-  float result = static_cast<float>(y);
+  return static_cast<float>(y);
+}
+
+__device__ __forceinline__ float expf_libm(float x, const uint64_t *table) {
+  const float result = expf_libm_core(x, table);
   // |x| >= 88, infinities and NaN: libm branches to these cases before the arithmetic above; here
   // they are selects after it (whatever the arithmetic made of such an x is discarded), which
   // keeps the instruction stream straight -- a taken branch per element costs more than the math.
@@ -139,6 +144,19 @@ __device__ __forceinline__ float expf_libm(float x, const uint64_t *table) {
   const float big = x > 0x1.62e42ep6f ? __builtin_inff() : (x < -0x1.9fe368p6f ? 0.0f : result);
   const float special = abstop >= 0x7f8u ? (ux == 0xff800000u ? 0.0f : x + x) : big;
   return abstop >= 0x42bu ? special : result;
+}
+
+// 1 / d for 1 <= d < 2^100, correctly rounded: the instruction sequence the compiler expands an f32
+// division into (reciprocal estimate, two refinements, a final correction), minus the operand scaling
+// and the special-case fix-up, neither of which does anything for a denominator in that range.
+__device__ __forceinline__ float reciprocal_of_moderate(float d) {
+  const float r = __builtin_amdgcn_rcpf(d);
+  const float e0 = __builtin_fmaf(-d, r, 1.0f);
+  const float r1 = __builtin_fmaf(e0, r, r);
+  const float res = __builtin_fmaf(-d, r1, 1.0f);
+  const float q1 = __builtin_fmaf(res, r1, r1);
+  const float res2 = __builtin_fmaf(-d, q1, 1.0f);
+  return __builtin_fmaf(res2, r1, q1);
 }
 
 struct SiluF32 {
@@ -150,8 +168,21 @@ struct SiluF32 {
     const float s = 1.0f / d; // correctly rounded IEEE division
     return s * x;
   }
+  // |x| < 64: exp(-x) is an ordinary number and so is 1 + exp(-x) < 2^93 -- the same five operations
+  // with no special case anywhere, so that the elements of a vector are independent straight-line
+  // chains the scheduler can interleave (the general form above costs a masked region per element).
+  static __device__ __forceinline__ bool moderate(float x) { return ((f2u(x) >> 20) & 0x7ffu) < 0x428u; }
+  __device__ __forceinline__ float one_moderate(float x) const {
+    const float e = expf_libm_core(-x, table);
+    const float d = e + 1.0f;
+    return reciprocal_of_moderate(d) * x;
+  }
   __device__ __forceinline__ u32x4 vec(u32x4 v) const {
-    return u32x4{f2u(one(u2f(v.x))), f2u(one(u2f(v.y))), f2u(one(u2f(v.z))), f2u(one(u2f(v.w)))};
+    const float x0 = u2f(v.x), x1 = u2f(v.y), x2 = u2f(v.z), x3 = u2f(v.w);
+    const bool all = moderate(x0) && moderate(x1) && moderate(x2) && moderate(x3);
+    if (__builtin_amdgcn_ballot_w64(!all) == 0) // uniform over the wavefront: no lane holds anything unusual
+      return u32x4{f2u(one_moderate(x0)), f2u(one_moderate(x1)), f2u(one_moderate(x2)), f2u(one_moderate(x3))};
+    return u32x4{f2u(one(x0)), f2u(one(x1)), f2u(one(x2)), f2u(one(x3))};
   }
   __device__ __forceinline__ void scalar(const void *in, void *out, int64_t i) const {
     static_cast<float *>(out)[i] = one(static_cast<const float *>(in)[i]);
@@ -167,9 +198,19 @@ template <io::Dt D> struct Silu16 {
   __device__ __forceinline__ u32x4 vec(u32x4 v) const {
     float f[E::kPerVec];
     E::unpack(v, f);
+    bool all = true;
 #pragma unroll
     for (int i = 0; i < E::kPerVec; ++i)
-      f[i] = f32.one(f[i]);
+      all = all && SiluF32::moderate(f[i]);
+    if (__builtin_amdgcn_ballot_w64(!all) == 0) {
+#pragma unroll
+      for (int i = 0; i < E::kPerVec; ++i)
+        f[i] = f32.one_moderate(f[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < E::kPerVec; ++i)
+        f[i] = f32.one(f[i]);
+    }
     return E::pack(f);
   }
   __device__ __forceinline__ void scalar(const void *in, void *out, int64_t i) const {

@@ -86,6 +86,17 @@ def test_silu_within_one_ulp(host, orc, stream):
     assert host.silu(stream, np.array([0.0], np.float32))[0] == 0.0
 
 
+def test_silu_same_bits_as_the_oracle_on_ordinary_inputs(host, orc, stream):
+    """|x| < 64 takes the kernel's straight-line form (exp without its special cases, the reciprocal
+    as an explicit refinement sequence): the same bits as libm's expf and an IEEE division, on every
+    f32 in [1, 2) (2^23 consecutive values) and on 8 Mi values spread over (-64, 64)."""
+    sweep = np.arange(0x3f800000, 0x40000000, dtype=np.uint32).view(np.float32)
+    spread = orc.fill_uniform(1 << 23, "f32", 77, -63.99, 63.99)
+    for name, x in (("every f32 in [1,2)", sweep), ("-every f32 in [1,2)", -sweep), ("uniform(-64,64)", spread)):
+        say("silu bit-exact: " + name)
+        assert np.array_equal(host.silu(stream, x).view(np.uint32), orc.silu_f32(x).view(np.uint32)), name
+
+
 def test_silu_benchmark_shape(host, orc, stream):
     x = orc.fill_uniform(512 * 640 * 20 * 15, "f32", 20251, -8.0, 8.0)
     got, ref = host.silu(stream, x), orc.silu_f32(x)
