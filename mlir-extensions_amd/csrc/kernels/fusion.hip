@@ -53,6 +53,29 @@ __device__ const LogfEntry kLogfTable[16] = {
     {0x1.886e6037841edp-1, 0x1.1058bc8a07ee1p-2},  {0x1.767dcf5534862p-1, 0x1.4043057b6ee09p-2},
 };
 
+// The arithmetic of logf on the bits of a positive normal number (libm's main path).
+__device__ __forceinline__ float logf_libm_core(uint32_t ix, const LogfEntry *table) {
+  const uint32_t tmp = ix - 0x3f330000u;
+  const int i = (tmp >> 19) & 15;
+  const int k = static_cast<int32_t>(tmp) >> 23;
+  const uint32_t iz = ix - (tmp & 0xff800000u);
+  const double invc = table[i].invc, logc = table[i].logc;
+  const double z = static_cast<double>(u2f(iz));
+  const double r = z * invc - 1.0;
+  const double y0 = logc + static_cast<double>(k) * 0x1.62e42fefa39efp-1;
+  const double r2 = r * r;
+  double y = 0x1.5575b0be00b6ap-2 * r + -0x1.ffffef20a4123p-2;
+  y = -0x1.00ea348b88334p-2 * r2 + y;
+  y = y * r2 + (y0 + r);
+  return static_cast<float>(y);
+}
+
+// Positive, normal, finite and not 1.0: what libm sends straight down its main path.
+__device__ __forceinline__ bool logf_ordinary(float x) {
+  const uint32_t ix = f2u(x);
+  return ix - 0x00800000u < 0x7f800000u - 0x00800000u && ix != 0x3f800000u;
+}
+
 __device__ __forceinline__ float logf_libm(float x, const LogfEntry *table) {
   uint32_t ix = f2u(x);
   if (ix == 0x3f800000u)
@@ -69,19 +92,7 @@ __device__ __forceinline__ float logf_libm(float x, const LogfEntry *table) {
     ix = f2u(x * 0x1p23f);      // subnormal: normalise
     ix -= 23u << 23;
   }
-  const uint32_t tmp = ix - 0x3f330000u;
-  const int i = (tmp >> 19) & 15;
-  const int k = static_cast<int32_t>(tmp) >> 23;
-  const uint32_t iz = ix - (tmp & 0xff800000u);
-  const double invc = table[i].invc, logc = table[i].logc;
-  const double z = static_cast<double>(u2f(iz));
-  const double r = z * invc - 1.0;
-  const double y0 = logc + static_cast<double>(k) * 0x1.62e42fefa39efp-1;
-  const double r2 = r * r;
-  double y = 0x1.5575b0be00b6ap-2 * r + -0x1.ffffef20a4123p-2;
-  y = -0x1.00ea348b88334p-2 * r2 + y;
-  y = y * r2 + (y0 + r);
-  return static_cast<float>(y);
+  return logf_libm_core(ix, table);
 }
 
 __device__ __forceinline__ void stage_table(LogfEntry *lds) {
@@ -91,14 +102,19 @@ __device__ __forceinline__ void stage_table(LogfEntry *lds) {
 }
 
 // the chains, on f32 values
+// kOrdinary: the caller has checked logf_ordinary() for the logarithm's argument in every lane of the
+// wavefront, so the chain is straight-line code (libm's special cases cost a masked region per element,
+// which keeps the f64 chains of a vector's elements from interleaving).
+template <bool kOrdinary = false>
 __device__ __forceinline__ float loop_chain(float a, float b, const LogfEntry *table) {
-  const float t1 = logf_libm(a, table);
+  const float t1 = kOrdinary ? logf_libm_core(f2u(a), table) : logf_libm(a, table);
   const float t2 = __builtin_fabsf(b);
   const float t3 = t1 + t2;
   return t3 - a;
 }
+template <bool kOrdinary = false>
 __device__ __forceinline__ float input_chain(float a, float b, const LogfEntry *table) {
-  const float t1 = logf_libm(b, table);
+  const float t1 = kOrdinary ? logf_libm_core(f2u(b), table) : logf_libm(b, table);
   const float t2 = __builtin_fabsf(a);
   return t1 + t2;
 }
@@ -136,9 +152,19 @@ __device__ __forceinline__ void loop_fusion_pass(const void *__restrict__ a, con
         float fa[E::kPerVec], fb[E::kPerVec];
         E::unpack(va[j], fa);
         E::unpack(vb[j], fb);
+        bool ordinary = true;
 #pragma unroll
         for (int i = 0; i < E::kPerVec; ++i)
-          fa[i] = loop_chain(fa[i], fb[i], table);
+          ordinary = ordinary && logf_ordinary(fa[i]);
+        if (__builtin_amdgcn_ballot_w64(!ordinary) == 0) { // uniform over the wavefront
+#pragma unroll
+          for (int i = 0; i < E::kPerVec; ++i)
+            fa[i] = loop_chain<true>(fa[i], fb[i], table);
+        } else {
+#pragma unroll
+          for (int i = 0; i < E::kPerVec; ++i)
+            fa[i] = loop_chain(fa[i], fb[i], table);
+        }
         store128<true>(E::pack(fa), po + j * kThreads + threadIdx.x);
       }
     } else {
@@ -188,13 +214,24 @@ __device__ __forceinline__ void input_fusion_cols(const void *__restrict__ a, co
         const int e = u * kThreads + tid;
         const int64_t r = r0 + e / kCols, c = c0 + e % kCols;
         const bool ok = r < rows && c < cols;
-        xa[u] = ok ? E::get(a, r * cols + c) : 1.0f;
-        xb[u] = ok ? E::get(b, r * cols + c) : 1.0f;
+        xa[u] = ok ? E::get(a, r * cols + c) : 2.0f; // positions outside the matrix: any ordinary value, never added
+        xb[u] = ok ? E::get(b, r * cols + c) : 2.0f;
       }
+      bool ordinary = true;
 #pragma unroll
       for (int u = 0; u < kPerLane; ++u)
-        if (r0 + (u * kThreads) / kCols < rows) // uniform: passes that lie wholly below the last row are skipped
-          t[u * kThreads + tid] = input_chain(xa[u], xb[u], table);
+        ordinary = ordinary && logf_ordinary(xb[u]);
+      if (__builtin_amdgcn_ballot_w64(!ordinary) == 0) { // uniform over the wavefront
+#pragma unroll
+        for (int u = 0; u < kPerLane; ++u)
+          if (r0 + (u * kThreads) / kCols < rows) // uniform: passes that lie wholly below the last row are skipped
+            t[u * kThreads + tid] = input_chain<true>(xa[u], xb[u], table);
+      } else {
+#pragma unroll
+        for (int u = 0; u < kPerLane; ++u)
+          if (r0 + (u * kThreads) / kCols < rows)
+            t[u * kThreads + tid] = input_chain(xa[u], xb[u], table);
+      }
       __syncthreads(); // the tile is complete; the other buffer was consumed before the previous barrier
       if (tid < kCols && c0 + tid < cols) {
         const int n = rows - r0 < kTileRows ? int(rows - r0) : kTileRows;
