@@ -17,6 +17,10 @@
  *       benchmarks/relu/relu_gpu.mlir.in:3-13            dims = {n}
  *   imex_silu_f32 / _f16 / _bf16   (in, out, n:i64)
  *       benchmarks/silu/silu_gpu.mlir.in:3-19            dims = {n}
+ *   imex_exp_f32                   (in, out, n:i64)                 out = expf(in), libm's
+ *       test/Integration/Dialect/XeGPU/WG/math_exp.mlir:49-62    dims = {n}
+ *   imex_maximum_f32               (a, b, out, n:i64)               out = maximumf(a, b): NaN if either is
+ *       test/Integration/Dialect/XeGPU/WG/arith_maximumf.mlir:51-66   dims = {n}
  *   imex_softmax_f32 / _f16 / _bf16 (in, out, rows:i64, cols:i64)
  *       benchmarks/softmax/softmax_gpu.mlir.in:4-44      dims = {rows, cols}
  *   imex_rowsum_f32                (in, out, rows:i64, cols:i64, init:f32)

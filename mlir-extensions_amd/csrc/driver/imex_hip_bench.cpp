@@ -131,6 +131,12 @@ std::vector<Workload> workloads() {
        {{Elem::F32, {16, 96, 96}, true, -1, 1}, {Elem::F32, {96, 96, 16}, false, 0, 0}}, {16, 96, 96}, 0,
        2.0 * 16 * 96 * 96 * 4, false},
       // the fused chains at the benchmark's own size (launch-bound) and at one that streams from HBM
+      {"exp_f32_256x256", "imex_exp_f32", {256 * 256},
+       {{Elem::F32, {256 * 256}, true, -0.5f, 0.5f}, {Elem::F32, {256 * 256}, false, 0, 0}}, {256 * 256}, 0,
+       2.0 * 256 * 256 * 4, false},
+      {"maximum_f32_256x256", "imex_maximum_f32", {256 * 256},
+       {{Elem::F32, {256 * 256}, true, -0.5f, 0.5f}, {Elem::F32, {256 * 256}, true, -0.5f, 0.5f},
+        {Elem::F32, {256 * 256}, false, 0, 0}}, {256 * 256}, 0, 3.0 * 256 * 256 * 4, false},
       {"loop_fusion_f32_512x1024", "imex_loop_fusion_f32", {512 * 1024},
        {{Elem::F32, {512 * 1024}, true, 0.5f, 3}, {Elem::F32, {512 * 1024}, true, -3, 3},
         {Elem::F32, {512 * 1024}, false, 0, 0}}, {512 * 1024}, 0, 3.0 * 512 * 1024 * 4, false},

@@ -1,4 +1,4 @@
-// Element-wise kernels: ReLU (f32 / f16 / bf16) and SiLU (f32).
+// Element-wise kernels: ReLU and SiLU (f32 / f16 / bf16), exp and maximum (f32).
 //
 // Reference op bodies: benchmarks/relu/relu_gpu.mlir.in:3-13 (cmpf ugt + select)
 // and benchmarks/silu/silu_gpu.mlir.in:3-19 (negf, exp, addf, divf, then mulf in
@@ -54,6 +54,52 @@ template <typename Op, int kElemBytes>
 __device__ __forceinline__ void stream_map(const void *in, void *out, int64_t n, Op op) {
   stream_map_impl<Op, kElemBytes, true>(in, out, n, op);
 }
+
+// Two inputs, one output, all of one shape: Op::one(a, b) on 32-bit elements.
+template <typename Op>
+__device__ __forceinline__ void stream_map2_b32(const uint32_t *__restrict__ a, const uint32_t *__restrict__ b,
+                                                uint32_t *__restrict__ out, int64_t n, Op op) {
+  constexpr int kVecsPerThread = 4;
+  constexpr int64_t kElemsPerBlock = int64_t(kThreads) * kVecsPerThread * 4;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+                         reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  for (int64_t base = int64_t(blockIdx.x) * kElemsPerBlock; base < n; base += int64_t(gridDim.x) * kElemsPerBlock) {
+    if (aligned && base + kElemsPerBlock <= n) {
+      const u32x4 *pa = reinterpret_cast<const u32x4 *>(a + base), *pb = reinterpret_cast<const u32x4 *>(b + base);
+      u32x4 *po = reinterpret_cast<u32x4 *>(out + base);
+      u32x4 va[kVecsPerThread], vb[kVecsPerThread];
+#pragma unroll
+      for (int j = 0; j < kVecsPerThread; ++j) {
+        va[j] = load128<true>(pa + j * kThreads + threadIdx.x);
+        vb[j] = load128<true>(pb + j * kThreads + threadIdx.x);
+      }
+#pragma unroll
+      for (int j = 0; j < kVecsPerThread; ++j)
+        store128<true>(u32x4{op.one(va[j].x, vb[j].x), op.one(va[j].y, vb[j].y), op.one(va[j].z, vb[j].z),
+                             op.one(va[j].w, vb[j].w)},
+                       po + j * kThreads + threadIdx.x);
+    } else {
+      for (int64_t i = base + threadIdx.x; i < base + kElemsPerBlock && i < n; i += kThreads)
+        out[i] = op.one(a[i], b[i]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// arith.maximumf (test/Integration/Dialect/XeGPU/WG/arith_maximumf.mlir:61): the larger operand,
+// +0 above -0, and NaN if either operand is NaN (the first NaN operand, quieted).  On the bit
+// patterns: a float's order is its sign-magnitude integer order.
+// ---------------------------------------------------------------------------
+struct MaximumF32 {
+  static __device__ __forceinline__ int32_t key(uint32_t u) { // monotone in the float's value, -0 below +0
+    return static_cast<int32_t>(u ^ ((static_cast<int32_t>(u) >> 31) & 0x7fffffff));
+  }
+  __device__ __forceinline__ uint32_t one(uint32_t a, uint32_t b) const {
+    const bool nanA = (a & 0x7fffffffu) > 0x7f800000u, nanB = (b & 0x7fffffffu) > 0x7f800000u;
+    const uint32_t larger = key(a) >= key(b) ? a : b;
+    return nanA ? (a | 0x00400000u) : (nanB ? (b | 0x00400000u) : larger);
+  }
+};
 
 // ---------------------------------------------------------------------------
 // ReLU.  "ugt" = unordered or greater than: x if x > 0 or x is NaN (payload
@@ -189,6 +235,24 @@ struct SiluF32 {
   }
 };
 
+// math.exp on f32 (test/Integration/Dialect/XeGPU/WG/math_exp.mlir:57): libm's expf, as the CPU
+// lowering the reference checks against calls it.  |x| < 64 in every lane: the arithmetic alone.
+struct ExpF32 {
+  const uint64_t *table;
+  __device__ __forceinline__ u32x4 vec(u32x4 v) const {
+    const float x0 = u2f(v.x), x1 = u2f(v.y), x2 = u2f(v.z), x3 = u2f(v.w);
+    const bool all = SiluF32::moderate(x0) && SiluF32::moderate(x1) && SiluF32::moderate(x2) && SiluF32::moderate(x3);
+    if (__builtin_amdgcn_ballot_w64(!all) == 0)
+      return u32x4{f2u(expf_libm_core(x0, table)), f2u(expf_libm_core(x1, table)), f2u(expf_libm_core(x2, table)),
+                   f2u(expf_libm_core(x3, table))};
+    return u32x4{f2u(expf_libm(x0, table)), f2u(expf_libm(x1, table)), f2u(expf_libm(x2, table)),
+                 f2u(expf_libm(x3, table))};
+  }
+  __device__ __forceinline__ void scalar(const void *in, void *out, int64_t i) const {
+    static_cast<float *>(out)[i] = expf_libm(static_cast<const float *>(in)[i], table);
+  }
+};
+
 // 16-bit SiLU: widen to f32, the same five f32 operations, one rounding back to the 16-bit type
 // (the policy the reference applies to 16-bit element types on the GPU,
 // docs/Transforms/BF16ToGpu.md:17-26; benchmarks/silu/silu.dtypes.in lists f16).
@@ -218,7 +282,7 @@ template <io::Dt D> struct Silu16 {
   }
 };
 
-// SiLU launch body: the 32-entry table staged in LDS (the index is data-dependent, and LDS serves
+// SiLU / exp launch body: the 32-entry table staged in LDS (the index is data-dependent, and LDS serves
 // 64 different addresses per access where a constant load would not); below 4 Mi elements a lane's
 // exponentials and divisions are the critical path, so one vector per lane and pass instead of four.
 template <typename Op, int kElemBytes, typename Make>
@@ -251,6 +315,15 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_relu_bf16(const uint
 
 extern "C" __global__ __launch_bounds__(kThreads) void imex_silu_f32(const float *in, float *out, int64_t n) {
   silu_launch<SiluF32, 4>(in, out, n, [](const uint64_t *table) { return SiluF32{table}; });
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_exp_f32(const float *in, float *out, int64_t n) {
+  silu_launch<ExpF32, 4>(in, out, n, [](const uint64_t *table) { return ExpF32{table}; });
+}
+
+extern "C" __global__ __launch_bounds__(kThreads) void imex_maximum_f32(const uint32_t *a, const uint32_t *b,
+                                                                       uint32_t *out, int64_t n) {
+  stream_map2_b32(a, b, out, n, MaximumF32{});
 }
 
 extern "C" __global__ __launch_bounds__(kThreads) void imex_silu_f16(const uint16_t *in, uint16_t *out,

@@ -45,6 +45,8 @@ const Entry kEntries[] = {
     {"imex_silu_f32", "(in: f32*, out: f32*, n: i64)", Module::Eltwise, Shape::Fusion32, 1},
     {"imex_silu_f16", "(in: f16*, out: f16*, n: i64)", Module::Eltwise, Shape::Fusion16, 1},
     {"imex_silu_bf16", "(in: bf16*, out: bf16*, n: i64)", Module::Eltwise, Shape::Fusion16, 1},
+    {"imex_exp_f32", "(in: f32*, out: f32*, n: i64)", Module::Eltwise, Shape::Fusion32, 1},
+    {"imex_maximum_f32", "(a: f32*, b: f32*, out: f32*, n: i64)", Module::Eltwise, Shape::Eltwise32, 1},
     {"imex_softmax_f32", "(in: f32*, out: f32*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows32, 2},
     {"imex_softmax_f16", "(in: f16*, out: f16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows16, 2},
     {"imex_softmax_bf16", "(in: bf16*, out: bf16*, rows: i64, cols: i64)", Module::Softmax, Shape::SoftmaxRows16, 2},

@@ -360,6 +360,16 @@ def _binary(stream, kernel, a, b, dtype, dims, out_shape):
             stream.free(p)
 
 
+def exp(stream, x):
+    """test/Integration/Dialect/XeGPU/WG/math_exp.mlir:57 (math.exp on f32: libm's expf)"""
+    return _unary(stream, "imex_exp_f32", x, "f32", [x.size])
+
+
+def maximum(stream, a, b):
+    """test/Integration/Dialect/XeGPU/WG/arith_maximumf.mlir:61 (arith.maximumf on f32)"""
+    return _binary(stream, "imex_maximum_f32", a, b, "f32", [a.size], a.shape)
+
+
 def loop_fusion(stream, a, b, dtype="f32"):
     """benchmarks/kLoopFusion/kLoopFusion.mlir.in:4-30: (log a + |b|) - a"""
     return _binary(stream, "imex_loop_fusion_" + dtype, a, b, dtype, [a.size], a.shape)

@@ -331,6 +331,22 @@ void oracle_logf_n(const float *in, float *out, size_t n) {
 
 float oracle_expf_cr(float x) { return (float)exp((double)x); }
 
+/* arith.maximumf, as the CPU loop of WG/arith_maximumf.mlir:122-129 applies it element by element:
+   IEEE-754 maximum -- NaN if either operand is NaN (the first one, quieted, is what x86 code
+   generation returns), +0 above -0. */
+void oracle_maximum_f32(const float *a, const float *b, float *out, size_t n) {
+  for (size_t i = 0; i < n; ++i) {
+    uint32_t ua, ub, r;
+    memcpy(&ua, &a[i], 4);
+    memcpy(&ub, &b[i], 4);
+    if (a[i] != a[i]) r = ua | 0x00400000u;
+    else if (b[i] != b[i]) r = ub | 0x00400000u;
+    else if (a[i] == b[i]) r = (ua & 0x80000000u) ? ub : ua; /* equal values: -0 only if both are */
+    else r = a[i] > b[i] ? ua : ub;
+    memcpy(&out[i], &r, 4);
+  }
+}
+
 void oracle_expf_n(const float *in, float *out, size_t n) {
   for (size_t i = 0; i < n; ++i) out[i] = expf(in[i]);
 }

@@ -32,6 +32,8 @@
  *   flash attention                                : the reference's own check input
  *       (every element 0.625 -> every output 0.625, flash_attention_fwd.mlir:481-485)
  *       and closed forms (one-hot scores, uniform scores = mean of V);
+ *   maximumf                                      : closed forms (order, signed zeros, NaN if either
+ *       operand is; which NaN comes back is parity unpinned -- the reference's test draws no NaN);
  *   loop fusion / input fusion chains             : parity unpinned by reference
  *       tests (the benchmarks feed constants and check nothing); pinned by closed
  *       forms against an f64 evaluation.
@@ -80,6 +82,7 @@ void oracle_flash_attention_rows(const uint16_t *Q, const uint16_t *K, const uin
                                  int64_t n_ctx, int64_t d_head, float sm_scale, const int64_t *rows,
                                  int64_t nrows); /* WG/flash_attention_fwd.mlir:332-421 */
 void oracle_logf_n(const float *in, float *out, size_t n);              /* the host libm logf the fused chains call */
+void oracle_maximum_f32(const float *a, const float *b, float *out, size_t n);   /* WG/arith_maximumf.mlir:122-129 (arith.maximumf) */
 float oracle_expf_cr(float x);                                          /* correctly rounded exp via f64 */
 void oracle_expf_n(const float *in, float *out, size_t n);              /* the host libm expf the oracle's silu/softmax call */
 

@@ -176,6 +176,20 @@ def silu_16(x, dtype):
     return y
 
 
+def expf_n(x):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().oracle_expf_n(_p(x), _p(out), C.c_size_t(x.size))
+    return out
+
+
+def maximum_f32(a, b):
+    a, b = _c(a, np.float32), _c(b, np.float32)
+    out = np.empty_like(a)
+    lib().oracle_maximum_f32(_p(a), _p(b), _p(out), C.c_size_t(a.size))
+    return out
+
+
 def loop_fusion_f32(a, b):
     a, b = _c(a, np.float32), _c(b, np.float32)
     out = np.empty_like(a)

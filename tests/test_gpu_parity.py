@@ -103,6 +103,35 @@ def test_silu_benchmark_shape(host, orc, stream):
     assert orc.ulp_distance_f32(got, ref).max() <= 1
 
 
+# ============================ exp, maximum ================================
+def test_exp_same_bits_as_libm(host, orc, stream):
+    """WG/math_exp.mlir: math.exp against the CPU loop's libm call -- the test's own input range
+    (-0.5, 0.5), the whole finite range, and the special values."""
+    for name, x in (("reference range", orc.fill_uniform(256 * 256, "f32", 31, -0.5, 0.5)),
+                    ("(-110, 110)", orc.fill_uniform(1 << 21, "f32", 32, -110.0, 110.0)),
+                    ("(-64, 64) ragged", orc.fill_uniform((1 << 20) + 13, "f32", 33, -63.9, 63.9))):
+        say("exp: " + name)
+        assert np.array_equal(host.exp(stream, x).view(np.uint32), orc.expf_n(x).view(np.uint32)), name
+    special = np.array([0.0, -0.0, np.inf, -np.inf, 88.72, 88.73, -103.9, -104.0, 1e-45, -1e-45, 1e38, -1e38, 64.0, -64.0],
+                       np.float32)
+    assert np.array_equal(host.exp(stream, special).view(np.uint32), orc.expf_n(special).view(np.uint32))
+    assert np.isnan(host.exp(stream, np.array([np.nan], np.float32))[0])
+
+
+def test_maximum_matches_the_oracle(host, orc, stream):
+    """WG/arith_maximumf.mlir: bit for bit where no operand is NaN, NaN where one is."""
+    a, b = orc.fill_uniform(256 * 256, "f32", 41, -0.5, 0.5), orc.fill_uniform(256 * 256, "f32", 42, -0.5, 0.5)
+    assert np.array_equal(host.maximum(stream, a, b), np.maximum(a, b))
+    n = (1 << 20) + 7
+    a, b = orc.fill_bits(n, "f32", 43).view(np.float32).copy(), orc.fill_bits(n, "f32", 44).view(np.float32).copy()
+    a[:8] = [0.0, -0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, np.nan]
+    b[:8] = [-0.0, 0.0, -0.0, 1.0, -1.0, 1.0, np.nan, np.nan]
+    got, ref = host.maximum(stream, a, b), orc.maximum_f32(a, b)
+    nan = np.isnan(ref)
+    assert np.array_equal(np.isnan(got), nan) and nan[5] and nan[6] and nan[7]
+    assert np.array_equal(got[~nan].view(np.uint32), ref[~nan].view(np.uint32))
+
+
 # =============================== Softmax ==================================
 def close_16(orc, got_bits, ref_bits, dtype):
     got, ref = orc.to_float(got_bits, dtype), orc.to_float(ref_bits, dtype)

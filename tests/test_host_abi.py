@@ -61,6 +61,8 @@ def test_launch_shapes(host):
     ls = host.launch_shape
     assert ls("imex_relu_f32", [4096 * 4096]) == ((4096, 1, 1), (256, 1, 1), 0)
     assert ls("imex_relu_f32", [1])[0] == (1, 1, 1)
+    assert ls("imex_maximum_f32", [256 * 256]) == ((16, 1, 1), (256, 1, 1), 0)
+    assert ls("imex_exp_f32", [256 * 256]) == ((64, 1, 1), (256, 1, 1), 0)  # one vector per lane below 4 Mi elements
     assert ls("imex_relu_f32", [0])[0][0] == 0  # nothing to launch
     assert ls("imex_relu_bf16", [8193])[0] == (2, 1, 1)
     assert ls("imex_softmax_f16", [16384, 1024])[0] == (4096, 1, 1)

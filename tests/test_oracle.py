@@ -161,6 +161,24 @@ def test_libm_expf_vs_correctly_rounded(orc):
     assert got[0] == np.float32(math.exp(float(x[0]))) or ulps[0] == 1
 
 
+def test_maximumf_closed_forms(orc):
+    """arith.maximumf (WG/arith_maximumf.mlir:126): the reference's test draws random values in
+    (-0.5, 0.5) and compares with its own CPU loop, so no vector exists; what the operation is
+    fixes these: the larger value, +0 above -0 whichever side it is on, infinities ordered like
+    numbers, NaN whenever either operand is NaN, and agreement with numpy's maximum elsewhere."""
+    inf, nan = np.float32(np.inf), np.float32(np.nan)
+    a = np.array([1.0, -2.0, 0.0, -0.0, -0.0, inf, -inf, nan, 3.0, nan, -1e-45, 5e-39], np.float32)
+    b = np.array([2.0, -3.0, -0.0, 0.0, -0.0, 1.0, -1.0, 1.0, nan, nan, 1e-45, -5e-39], np.float32)
+    got = orc.maximum_f32(a, b)
+    want = np.array([2.0, -2.0, 0.0, 0.0, -0.0, inf, -1.0, nan, nan, nan, 1e-45, 5e-39], np.float32)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))  # bit patterns: signed zeros included
+    x, y = orc.fill_uniform(10000, "f32", 5, -0.5, 0.5), orc.fill_uniform(10000, "f32", 6, -0.5, 0.5)
+    assert np.array_equal(orc.maximum_f32(x, y), np.maximum(x, y))
+    assert np.array_equal(orc.maximum_f32(x, y), orc.maximum_f32(y, x))
+
+
 # ---- fused element-wise chains ------------------------------------------------------
 def test_libm_logf_vs_correctly_rounded(orc):
     """The host libm logf the fused chains call is within 1 ulp of the correctly
