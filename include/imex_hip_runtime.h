@@ -112,6 +112,8 @@ void mgpuLaunchKernel(void *kernel, size_t gridX, size_t gridY, size_t gridZ, si
 void *mgpuMemAlloc(size_t size, void *stream, int isShared);
 void mgpuMemFree(void *stream, void *ptr);
 void mgpuMemcpy(void *dst, void *src, size_t bytes, void *stream);
+/* `count` 32-bit words of `value`.  Runs as a kernel of this library (not as a memset on the stream), so a
+ * caller that captures the stream into a HIP graph gets an ordinary kernel node. */
 void mgpuMemset32(void *dst, unsigned int value, size_t count, void *stream);
 void *mgpuModuleLoad(const void *data, size_t dataSize);
 void *mgpuModuleGetFunction(void *module, const char *name);

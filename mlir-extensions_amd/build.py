@@ -77,9 +77,19 @@ def build_kernel_library(verbose=False):
 
 
 def build_runtime(verbose=False):
+    os.makedirs(LIB_DIR, exist_ok=True)
+    os.makedirs(BUILD_DIR, exist_ok=True)
+    # the library's own device code (the fill kernel behind mgpuMemset32), embedded like the kernel blobs
+    fill = os.path.join(LIB_DIR, "imex_runtime_fill.hsaco")
+    _run([HIPCC] + DEVICE_FLAGS + [os.path.join(CSRC, "runtime", "fill.hip"), "-o", fill], verbose)
+    stub = os.path.join(BUILD_DIR, "imex_runtime_blobs.S")
+    with open(stub, "w") as f:
+        f.write('  .section .rodata\n  .balign 4096\n  .global imex_runtime_fill_blob\nimex_runtime_fill_blob:\n')
+        f.write('  .incbin "%s"\n  .global imex_runtime_fill_blob_end\nimex_runtime_fill_blob_end:\n' % fill)
+        f.write('  .section .note.GNU-stack,"",@progbits\n')
     out = os.path.join(LIB_DIR, "libimex-hip-runtime.so")
     srcs = [os.path.join(CSRC, "runtime", "HipRuntimeWrappers.cpp"),
-            os.path.join(CSRC, "runtime", "ProfilerStats.cpp")]
+            os.path.join(CSRC, "runtime", "ProfilerStats.cpp"), stub]
     _run(["g++"] + HOST_FLAGS + ["-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(ROCM, "include"),
                                  "-shared", "-o", out] + srcs +
          ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib")], verbose)

@@ -29,6 +29,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -584,11 +585,26 @@ extern "C" void mgpuMemcpy(void *dst, void *src, size_t bytes, void *stream) {
   catchAll([&]() { copyMemory(stream ? asQueue(stream) : defaultQueue(), dst, src, bytes); });
 }
 
+// The fill kernel this library carries (csrc/runtime/fill.hip), embedded at build time.
+extern "C" const char imex_runtime_fill_blob[], imex_runtime_fill_blob_end[];
+
+// A kernel launch, not a memset on the stream: memset nodes recorded into a captured HIP graph
+// have replayed wrongly on this platform, and the queue may sit on a stream its owner captures.
 extern "C" void mgpuMemset32(void *dst, unsigned int value, size_t count, void *stream) {
   catchAll([&]() {
     GpuHipQueue *q = stream ? asQueue(stream) : defaultQueue();
+    if (count == 0)
+      return;
     CHECK_HIP(hipSetDevice(q->device));
-    CHECK_HIP(hipMemsetD32Async(reinterpret_cast<hipDeviceptr_t>(dst), static_cast<int>(value), count, q->stream));
+    hipModule_t module =
+        loadModule(q, imex_runtime_fill_blob, size_t(imex_runtime_fill_blob_end - imex_runtime_fill_blob));
+    hipFunction_t fill = getKernel(module, "imex_runtime_fill_b32");
+    uint32_t word = value;
+    int64_t n = static_cast<int64_t>(count);
+    void *params[] = {&dst, &word, &n};
+    const size_t perGroup = 256 * 4 * 4; // 256 lanes, about four 16-byte stores each
+    const unsigned groups = static_cast<unsigned>(std::min<size_t>((count + perGroup - 1) / perGroup, 2048));
+    CHECK_HIP(hipModuleLaunchKernel(fill, groups, 1, 1, 256, 1, 1, 0, q->stream, params, nullptr));
   });
 }
 

@@ -1,0 +1,27 @@
+// The runtime library's own device code: a 32-bit pattern fill.
+//
+// mgpuMemset32 (lib/ExecutionEngine/LEVELZERORUNTIME/LevelZeroRuntimeWrappers.cpp:705-711, the
+// upstream gpu.memset lowering) runs this kernel instead of recording a memset on the stream,
+// so that a caller who captures the stream into a HIP graph gets an ordinary kernel node.
+//
+// Launch: block (256,1,1), any grid (workgroups stride over the buffer).
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+extern "C" __global__ __launch_bounds__(256) void imex_runtime_fill_b32(uint32_t *dst, uint32_t value, int64_t n) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const int64_t tid = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t threads = int64_t(gridDim.x) * 256;
+  // words before the first 16-byte boundary, then whole vectors, then the tail
+  const int64_t head = min(n, int64_t((16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15) / 4);
+  const int64_t vecs = (n - head) / 4;
+  for (int64_t i = tid; i < head; i += threads)
+    dst[i] = value;
+  u32x4 *body = reinterpret_cast<u32x4 *>(dst + head);
+  const u32x4 v = {value, value, value, value};
+  for (int64_t i = tid; i < vecs; i += threads)
+    body[i] = v;
+  for (int64_t i = head + vecs * 4 + tid; i < n; i += threads)
+    dst[i] = value;
+}

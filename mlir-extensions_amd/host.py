@@ -204,6 +204,10 @@ class Stream:
     def free(self, ptr):
         self.rt.gpuMemFree(self.handle, int(ptr))
 
+    def fill32(self, ptr, value, count):
+        """mgpuMemset32 on this queue: `count` 32-bit words of `value`."""
+        self.rt.mgpuMemset32(int(ptr), value, count, self.handle)
+
     def copy(self, dst, src, nbytes):
         self.rt.gpuMemCopy(self.handle, int(dst), int(src), nbytes)
 

@@ -226,26 +226,34 @@ def test_adopted_stream_and_graph_replay(host, orc):
     d_a, d_b, d_t, d_o = s.to_device(a), s.to_device(b), s.alloc(n * 4), s.alloc(n * 4)
     chain = s.prepare("imex_loop_fusion_f32", [n], [d_a, d_b, d_t, n])
     relu = s.prepare("imex_relu_f32", [n], [d_t, d_o, n])
+    d_m = s.alloc(n * 4 + 4)
+    marks = int(d_m) + 4, 0x3fc00000, n - 3     # a fill that starts and ends off the 16-byte grid
     chain(), relu()   # eager once: modules loaded, kernels resolved, nothing left to allocate under capture
+    s.fill32(*marks)
     s.wait()
     want = orc.relu_f32(orc.loop_fusion_f32(a, b))
     assert np.array_equal(s.from_device(d_o, (n,), np.float32).view(np.uint32), want.view(np.uint32))
 
     graph, exe = C.c_void_p(), C.c_void_p()
     assert hip.hipStreamBeginCapture(raw, 2) == 0          # relaxed mode
+    s.fill32(*marks)                                        # the fill is a kernel, so an ordinary graph node
     chain(), relu()
     assert hip.hipStreamEndCapture(raw, C.byref(graph)) == 0
     assert hip.hipGraphInstantiate(C.byref(exe), graph, None, None, C.c_size_t(0)) == 0
     for seed in (203, 204, 205):
         a2 = orc.fill_uniform(n, "f32", seed, 0.5, 3.0)
         s.copy(d_a, a2.ctypes.data, n * 4)                  # new input, same buffers
-        s.copy(d_o, np.zeros(n, np.float32).ctypes.data, n * 4)
+        zeros, stale = np.zeros(n, np.float32), np.full(n + 1, seed, np.uint32)  # named: alive until copied
+        s.copy(d_o, zeros.ctypes.data, n * 4)
+        s.copy(d_m, stale.ctypes.data, n * 4 + 4)
         assert hip.hipGraphLaunch(exe, raw) == 0
         s.wait()
+        filled = s.from_device(d_m, (n + 1,), np.uint32)
+        assert filled[0] == seed and np.all(filled[1:n - 2] == 0x3fc00000) and np.all(filled[n - 2:] == seed), seed
         got = s.from_device(d_o, (n,), np.float32)
         assert np.array_equal(got.view(np.uint32), orc.relu_f32(orc.loop_fusion_f32(a2, b)).view(np.uint32)), seed
     assert hip.hipGraphExecDestroy(exe) == 0 and hip.hipGraphDestroy(graph) == 0
-    for p in (d_a, d_b, d_t, d_o):
+    for p in (d_a, d_b, d_t, d_o, d_m):
         s.free(p)
     s.close()                                               # must leave the adopted stream alive
     assert hip.hipStreamSynchronize(raw) == 0
