@@ -173,10 +173,11 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
   case Shape::SoftmaxRows32:
   case Shape::SoftmaxRows16: {
     // Rows of up to 128 x 16 B stay in registers, one per wavefront (four per
-    // workgroup); longer rows take a workgroup each.  The kernel strides over
+    // workgroup; two per wavefront from 16384 rows on); longer rows take a workgroup each.  The kernel strides over
     // the rows, so any grid is correct; this one covers them in a single pass.
     const int64_t regCols = e->shape == Shape::SoftmaxRows16 ? 1024 : 512;
-    grid[0] = dims[1] <= regCols ? ceilDiv(dims[0], 4) : static_cast<size_t>(dims[0] < 1048560 ? dims[0] : 1048560);
+    grid[0] = dims[1] <= regCols ? ceilDiv(dims[0], dims[0] >= 16384 ? 8 : 4)
+                                 : static_cast<size_t>(dims[0] < 1048560 ? dims[0] : 1048560);
     if (dims[1] == 0)
       grid[0] = 0;
     break;

@@ -159,7 +159,8 @@ def test_softmax_config_f16_16384x1024(host, orc, stream):
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 1), (3, 7), (5, 8), (16, 2000), (64, 2000), (7, 1000), (9, 512), (4, 4096),
-                                       (3, 5000), (2, 65536 + 8), (1025, 64), (6, 1016)])
+                                       (3, 5000), (2, 65536 + 8), (1025, 64), (6, 1016),
+                                       (16385, 24), (20001, 8)])  # two rows per wavefront, odd row counts
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 def test_softmax_shapes(host, orc, stream, rows, cols, dtype):
     say("softmax %s %dx%d" % (dtype, rows, cols))
