@@ -133,6 +133,11 @@ struct BiasAccumulateF32 { // C = bias[n] + (C + acc)  (bias.mlir:88-94,112-113)
 // the result is rounded to bf16, 2^-9 relative, straight afterwards.
 __device__ __forceinline__ float silu_fast(float v) { return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
 
+// f32 -> bf16 by the hardware's conversion (round to nearest even; pairs become one v_cvt_pk_bf16_f32).
+// Numbers convert as float_to_bf16_bits does; a NaN keeps its leading payload bits instead of becoming
+// the canonical one.
+__device__ __forceinline__ uint16_t bf16_bits_hw(float f) { return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f)); }
+
 struct BiasSiluBF16 {   // out = bf16( silu( acc + bias[n] ) )
   static constexpr bool kColumnsInRegisters = true;
   uint16_t *out;
@@ -140,7 +145,7 @@ struct BiasSiluBF16 {   // out = bf16( silu( acc + bias[n] ) )
   __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
     const float v = acc + bias[n];
     const float y = silu_fast(v);
-    out[m * N + n] = static_cast<uint16_t>(float_to_bf16_bits(y));
+    out[m * N + n] = bf16_bits_hw(y);
   }
   __device__ __forceinline__ void vec4(int64_t m, int64_t n, int64_t N, f32x4 acc) const {
     const f32x4 b = *reinterpret_cast<const f32x4u *>(bias + n);
@@ -149,7 +154,7 @@ struct BiasSiluBF16 {   // out = bf16( silu( acc + bias[n] ) )
     for (int r = 0; r < 4; ++r) {
       const float v = acc[r] + b[r];
       const float y = silu_fast(v);
-      o[r] = static_cast<uint16_t>(float_to_bf16_bits(y));
+      o[r] = bf16_bits_hw(y);
     }
     *reinterpret_cast<u16x4u *>(out + m * N + n) = o;
   }
