@@ -192,10 +192,12 @@ __device__ __forceinline__ void loop_fusion(const void *__restrict__ a, const vo
 // and walks the rows in tiles of 4096 / kCols: all 256 lanes evaluate the chain of a tile into
 // LDS (coalesced along the rows), then lane j < kCols adds column j's values of the tile to its
 // running sum, in row order.  The tile is double-buffered, so the ordered additions of one tile
-// run under the loads and logarithms of the next, with one barrier per tile.
-constexpr int kTileElems = 4096;
+// run under the loads and logarithms of the next, with one barrier per tile.  Short matrices
+// (up to 1024 rows, the reference's 512 x 1024 among them) use tiles of 1024 elements, so that
+// there is a next tile to overlap with; tall ones are faster with fewer barriers.
+constexpr int kTileElems = 4096, kSmallTileElems = 1024;
 
-template <Dt D, int kCols>
+template <Dt D, int kCols, int kTileElems = ::kTileElems>
 __device__ __forceinline__ void input_fusion_cols(const void *__restrict__ a, const void *__restrict__ b,
                                                   void *__restrict__ out, int64_t rows, int64_t cols,
                                                   const LogfEntry *table, float *tile) {
@@ -284,7 +286,12 @@ __device__ __forceinline__ void input_fusion(const void *__restrict__ a, const v
   case 32: input_fusion_cols<D, 32>(a, b, out, rows, cols, table, tile); break;
   case 16: input_fusion_cols<D, 16>(a, b, out, rows, cols, table, tile); break;
   case 8: input_fusion_cols<D, 8>(a, b, out, rows, cols, table, tile); break;
-  default: input_fusion_cols<D, 4>(a, b, out, rows, cols, table, tile); break;
+  default:
+    if (rows <= 1024)
+      input_fusion_cols<D, 4, kSmallTileElems>(a, b, out, rows, cols, table, tile);
+    else
+      input_fusion_cols<D, 4>(a, b, out, rows, cols, table, tile);
+    break;
   }
 }
 
