@@ -298,12 +298,14 @@ def gemm(a, b, ab_dtype, c=None, out_round="f32"):
     return out
 
 
-def gemm_rows(a, b, rows, ab_dtype):
+def gemm_rows(a, b, rows, ab_dtype, c0_rows=None):
+    """Rows `rows` of C0 + A.B (the i-k-j loop accumulates onto what C holds); C0 = 0 when not given."""
     a, b = _c(a), _c(b)
     K = a.shape[1]
     N = b.shape[1]
     rows = np.ascontiguousarray(rows, np.int64)
-    out = np.zeros((rows.size, N), np.float32)
+    out = np.zeros((rows.size, N), np.float32) if c0_rows is None else _c(c0_rows, np.float32).copy()
+    assert out.shape == (rows.size, N)
     lib().oracle_gemm_rows(_p(a), _p(b), _p(out), _p(rows), C.c_int64(rows.size), C.c_int64(N), C.c_int64(K),
                            DT[ab_dtype])
     return out

@@ -186,6 +186,30 @@ def test_softmax_bf16_and_exact_rows(host, orc, stream):
     assert np.all(got[:, 5] == 1.0) and got.sum() == 4.0
 
 
+@pytest.mark.parametrize("dtype,cols", [("f32", 20), ("f32", 512), ("f16", 1024), ("f32", 3000), ("f16", 4096),
+                                        ("f32", 5000), ("f16", 70000)])
+def test_softmax_nan_and_infinite_rows(host, orc, stream, dtype, cols):
+    """Rows the benchmark's inputs never hold, on every path of the kernel (registers, LDS, streamed):
+    a NaN anywhere makes its whole row NaN (arith.maximumf and the sum both carry it), a row of
+    nothing but -inf is 0/0 = NaN because the running maximum starts at -3.40282347e38 rather than
+    -inf, +inf in a row gives inf - inf = NaN, and a -inf among finite values is an exact zero."""
+    say("softmax special rows %s cols=%d" % (dtype, cols))
+    x = orc.to_float(orc.fill_normal(6 * cols, dtype, 71, 0.0, 2.0), dtype).reshape(6, cols).copy()
+    x[1, cols // 3] = np.nan
+    x[2, :] = -np.inf
+    x[3, cols - 1] = np.inf
+    x[4, 0] = -np.inf
+    x[5, :] = -3.0e38 if dtype == "f32" else -65504.0
+    xin = x if dtype == "f32" else orc.from_float(x, dtype)
+    got = orc.to_float(host.softmax(stream, xin, dtype), dtype)
+    ref = orc.softmax_f32(x) if dtype == "f32" else orc.to_float(orc.softmax_16(xin, dtype), dtype)
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    assert np.isnan(ref[1]).all() and np.isnan(ref[2]).all() and np.isnan(ref[3]).all() and not np.isnan(ref[[0, 4, 5]]).any()
+    assert got[4, 0] == 0.0
+    ok = ~np.isnan(ref)
+    assert np.all(np.abs(got[ok] - ref[ok]) <= 1e-3 * np.abs(ref[ok]) + (2.0 ** -24 if dtype == "f16" else 0.0))
+
+
 # =============================== Reductions ================================
 def test_rowsum_golden_and_exact(host, orc, stream):
     g = GOLD["sum_f32_10x20"]
@@ -822,24 +846,114 @@ def test_gemm_transposed_operands(host, orc, stream, which):
     assert np.max(np.abs(fixed - (c0 + got))) <= 1e-4
 
 
+def _launch_raw(host, stream, name, args, grid, block=(512, 1, 1)):
+    """gpuLaunchKernel with an explicit launch shape (the reference's own, for the fixed-shape entries)."""
+    import ctypes as C
+    fn = stream.kernel(name)
+    descs, keep = host._pack_params(args)
+    stream.rt.gpuLaunchKernel(stream.handle, fn, grid[0], grid[1], grid[2], block[0], block[1], block[2], 0,
+                              C.cast(descs, C.c_void_p), None)
+    stream.wait()
+    del keep
+
+
+def _column_checksum_f64(a_f32, b_f32):
+    """(1^T A) B in f64, in column panels so that B is never held whole as f64."""
+    s = a_f32.sum(axis=0, dtype=np.float64)
+    out = np.empty(b_f32.shape[1], np.float64)
+    for n0 in range(0, b_f32.shape[1], 1024):
+        out[n0:n0 + 1024] = s @ b_f32[:, n0:n0 + 1024].astype(np.float64)
+    return out
+
+
+STRIDED_ROWS_4096 = np.array(sorted(set(list(range(0, 4096, 97)) + [1, 127, 128, 255, 256, 2047, 2048, 4095])))
+
+
 def test_gemm_config_mlp_bf16_bias_silu(host, orc, stream):
     M, K, N = 4096, 4096, 11008
     a = orc.fill_normal(M * K, "bf16", 20248, 0.0, 1.0).reshape(M, K)
     b = orc.fill_normal(K * N, "bf16", 20249, 0.0, 0.02).reshape(K, N)
     bias = orc.fill_normal(N, "f32", 20250, 0.0, 0.1)
     got = orc.bfloat_to_float(host.gemm_bias_silu(stream, a, b, bias))
-    rows = np.array([0, 1, 255, 256, 1000, 2047, 2048, 3333, 4095])
-    ref = orc.bfloat_to_float(orc.bias_silu_bf16(orc.gemm_rows(a, b, rows, "bf16"), bias))
+    rows = STRIDED_ROWS_4096  # a stride of 97 lands in every 128-row wavefront block of every 256-row tile
+    acc = orc.gemm_rows(a, b, rows, "bf16")
+    ref = orc.bfloat_to_float(orc.bias_silu_bf16(acc, bias))
     err = np.max(np.abs(got[rows] - ref)) / np.max(np.abs(ref))
-    say("mlp gemm: max|d|/max|ref| = %.3e" % err)
+    say("mlp gemm: max|d|/max|ref| = %.3e over %d rows" % (err, rows.size))
     assert err <= 5e-3
     # element-wise: within one bf16 step wherever the value is not tiny
     big = np.abs(ref) > 1e-2
     assert np.max(np.abs(got[rows][big] - ref[big]) / np.abs(ref[big])) <= 2.0 ** -7
-    # plain bf16 GEMM with f32 output against the same rows
+    # plain bf16 GEMM with f32 output: the same rows, and every column's sum against (1^T A) B in f64
     plain = host.gemm(stream, a, b, ab_dtype="bf16")
-    ref32 = orc.gemm_rows(a, b, rows, "bf16")
-    assert gemm_close(plain[rows], ref32)
+    assert gemm_close(plain[rows], acc)
+    want = _column_checksum_f64(orc.bfloat_to_float(a), orc.bfloat_to_float(b))
+    assert np.max(np.abs(plain.sum(axis=0, dtype=np.float64) - want)) <= 1e-3 * np.max(np.abs(want)) + 0.05
+    # the whole fused output against the epilogue applied (in f64) to that checked f32 product:
+    # every element within one bf16 step, so no tile, wavefront block or column strip is left out
+    v = plain.astype(np.float64) + bias.astype(np.float64)[None, :]
+    want = v / (1.0 + np.exp(-v))
+    del v
+    d = np.abs(got - want)
+    assert np.all(d <= 2.0 ** -7 * np.abs(want) + 1e-6), "fused epilogue differs at %s" % (np.argwhere(d > 2.0 ** -7 * np.abs(want) + 1e-6)[:4],)
+
+
+def test_gemm_reference_bias_kernel_4096(host, orc, stream):
+    """WG/gemm_4kx4kx4k_f16_f16_f32_bias.mlir:77-116: kernel arguments (bias, C, A, B), grid 16 x 16,
+    C = bias[n] + (C + A.B); checked as the test itself does (:160-172): the f32 GEMM onto the initial C,
+    then C_ref[i,j] += bias[j].  The initial C is not zero here, so the accumulate is visible."""
+    M = N = K = 4096
+    a = orc.fill_uniform(M * K, "f16", 61, -0.5, 0.5).reshape(M, K)
+    b = orc.fill_uniform(K * N, "f16", 62, -0.5, 0.5).reshape(K, N)
+    c0 = orc.fill_uniform(M * N, "f32", 63, -1.0, 1.0).reshape(M, N)
+    bias = orc.fill_uniform(N, "f32", 64, -1.0, 1.0)
+    d_bias, d_c, d_a, d_b = (stream.to_device(t) for t in (bias, c0, a, b))
+    try:
+        _launch_raw(host, stream, "imex_gemm_4kx4kx4k_f16_f16_f32_bias", [d_bias, d_c, d_a, d_b], (16, 16, 1))
+        got = stream.from_device(d_c, (M, N), np.float32)
+        assert np.array_equal(stream.from_device(d_bias, (N,), np.float32), bias)
+    finally:
+        for p in (d_bias, d_c, d_a, d_b):
+            stream.free(p)
+    rows = STRIDED_ROWS_4096
+    # oracle: the i-k-j loop accumulates onto C0's rows, then the bias loop
+    ref = orc.bias_add_rows(orc.gemm_rows(a, b, rows, "f16", c0_rows=c0[rows]), bias)
+    err = np.max(np.abs(got[rows] - ref)) / np.max(np.abs(ref))
+    say("bias gemm 4096^3: max|d|/max|ref| = %.3e over %d rows" % (err, rows.size))
+    assert err <= 5e-3
+    assert orc.allclose_f32(got[rows], ref)  # the reference's own check (atol 1e-4, rtol 1e-3)
+    # every column: 1^T C = (1^T A) B + 1^T C0 + M bias[n], in f64
+    want = (_column_checksum_f64(orc.half_to_float(a), orc.half_to_float(b)) + c0.sum(axis=0, dtype=np.float64)
+            + M * bias.astype(np.float64))
+    assert np.max(np.abs(got.sum(axis=0, dtype=np.float64) - want)) <= 1e-3 * np.max(np.abs(want)) + 0.05
+    # and every element against the accumulate kernel plus the bias (two roundings apart at most)
+    acc = host.gemm(stream, a, b, c=c0, ab_dtype="f16")
+    assert np.max(np.abs(got - (acc + bias[None, :]))) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype,M,N,K", [("bf16", 512, 512, 96), ("bf16", 300, 520, 1024), ("f16", 768, 256, 4096)])
+def test_gemm_tiled_accumulate_integers_exact(host, orc, stream, dtype, M, N, K):
+    """C += A.B on the MFMA path with integer operands and an integer C0: exact in any order."""
+    a = orc.fill_int(M * K, dtype, 41, -4, 4).reshape(M, K)
+    b = orc.fill_int(K * N, dtype, 42, -4, 4).reshape(K, N)
+    c0 = orc.fill_int(M * N, "f32", 43, -1000, 1000).reshape(M, N)
+    want = orc.to_float(a, dtype).astype(np.int64) @ orc.to_float(b, dtype).astype(np.int64) + c0.astype(np.int64)
+    got = host.gemm(stream, a, b, c=c0, ab_dtype=dtype)
+    assert np.array_equal(got.astype(np.int64), want)
+
+
+def test_gemm_f16_output_4096(host, orc, stream):
+    """WG/gemm_4kx4kx4k_f16_f16_f16.mlir at its own size: f32 accumulation, one rounding to f16."""
+    M = N = K = 4096
+    a = orc.fill_uniform(M * K, "f16", 65, -0.5, 0.5).reshape(M, K)
+    b = orc.fill_uniform(K * N, "f16", 66, -0.5, 0.5).reshape(K, N)
+    got = orc.half_to_float(host.gemm(stream, a, b, ab_dtype="f16", out_dtype="f16"))
+    rows = STRIDED_ROWS_4096
+    ref = orc.half_to_float(orc.float_to_half(orc.gemm_rows(a, b, rows, "f16")))
+    assert gemm_close(got[rows], ref)
+    want = _column_checksum_f64(orc.half_to_float(a), orc.half_to_float(b))
+    # 4096 roundings to f16 per column, each below 2^-11 relative
+    assert np.max(np.abs(got.sum(axis=0, dtype=np.float64) - want)) <= 2e-3 * np.max(np.abs(want)) + 0.5
 
 
 def test_gemm_f16_output_variant(host, orc, stream):

@@ -415,6 +415,10 @@ def test_gemm_closed_forms(orc):
     full = orc.gemm(a, b, "f16")
     rows = np.array([0, 5, 63])
     assert np.array_equal(orc.gemm_rows(a, b, rows, "f16"), full[rows])
+    # ... also onto a non-zero C (the reference loads C as the initial accumulator)
+    c0 = orc.fill_uniform(64 * 32, "f32", 9, -1, 1).reshape(64, 32)
+    assert np.array_equal(orc.gemm_rows(a, b, rows, "f16", c0_rows=c0[rows]), orc.gemm(a, b, "f16", c=c0)[rows])
+    assert orc.gemm(a, b, "f16", c=c0)[3, 9] != full[3, 9]
     # k-ascending f32 accumulation with a rounded product: compare with a literal loop
     af, bf = orc.half_to_float(a), orc.half_to_float(b)
     acc = np.float32(0)
