@@ -33,6 +33,10 @@ METRIC = "GEMM TFLOP/s (% MFMA peak) + softmax/reduce/transpose GB/s (% HBM peak
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X published dense f16 / bf16 MFMA rate
 FLUSH_BYTES = 512 << 20     # > L2 (8 x 4 MiB) + 256 MiB Infinity Cache
+SETTLE_LAUNCHES = 300       # untimed launches of the headline kernel before the caller's warm-up and timed steps
+# the reference's CPU benchmark templates (benchmarks/relu/relu_cpu.mlir.in:22-61): warm-ups, then wall-clocked calls
+# that allocate their result inside the timed call, average reported
+CPU_PROTOCOL = "full tensor, %d warm-ups + %d timed calls, result allocated inside each call, one core"
 
 
 def log(msg):
@@ -157,11 +161,12 @@ def build_workloads(host, orc, stream, only):
         b = gen_normal(K * N, "bf16", 20249, 0.0, 0.02).reshape(K, N)
         bias = gen_normal(N, "f32", 20250, 0.0, 0.1)
         cur.args = [dev(a), dev(b), dev(bias), out(M * N * 2), M, N, K]
-        rows = 64
+        rows = 512
 
-        def cpu(a=a, b=b, rows=rows):
-            ms = orc.time_gemm_rows(a, b, rows, "bf16")
-            return 2.0 * rows * N * K / (ms * 1e9), "first %d of 4096 rows, GEMM loop only" % rows
+        def cpu(a=a, b=b, bias=bias, rows=rows):
+            ms = orc.time_mlp_rows(a, b, bias, rows)
+            return 2.0 * rows * N * K / (ms * 1e9), ("first %d of 4096 rows: the i-k-j GEMM loop, then bias + SiLU + rounding "
+                                                     "to bf16; one un-warmed call" % rows)
         cur.cpu = cpu
         wl.append(cur)
 
@@ -171,7 +176,7 @@ def build_workloads(host, orc, stream, only):
                        "relu f32 [4096,4096] uniform(-1,1) seed 20241, out of place")
         x = gen_uniform(n, "f32", 20241, -1.0, 1.0)
         cur.args = [dev(x), out(n * 4), n]
-        cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_relu_f32(x, 2, 10) * 1e6), "full tensor, 2 warm-ups + 10 timed calls")
+        cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_relu_f32(x, 5, 200) * 1e6), CPU_PROTOCOL % (5, 200))
         wl.append(cur)
 
     if want("softmax_f16"):
@@ -180,7 +185,7 @@ def build_workloads(host, orc, stream, only):
                        "softmax f16 [16384,1024] normal(0,2) seed 20242, f32 internals")
         x = gen_normal(rows * cols, "f16", 20242, 0.0, 2.0).reshape(rows, cols)
         cur.args = [dev(x), out(rows * cols * 2), rows, cols]
-        cur.cpu = lambda x=x: (2.0 * x.size * 2 / (orc.time_softmax_f16(x, 1, 3) * 1e6), "full tensor, 1 warm-up + 3 timed calls")
+        cur.cpu = lambda x=x: (2.0 * x.size * 2 / (orc.time_softmax_f16(x, 5, 100) * 1e6), CPU_PROTOCOL % (5, 100))
         wl.append(cur)
 
     if want("rowsum_f32"):
@@ -189,7 +194,7 @@ def build_workloads(host, orc, stream, only):
                        "f32", "row-sum f32 [8192,8192] uniform(0,1) seed 20243 -> [8192]")
         x = gen_uniform(rows * cols, "f32", 20243, 0.0, 1.0).reshape(rows, cols)
         cur.args = [dev(x), out(rows * 4), rows, cols, 0.0]
-        cur.cpu = lambda x=x: ((x.size * 4.0 + x.shape[0] * 4.0) / (orc.time_rowsum_f32(x, 1, 5) * 1e6), "full tensor, 1 warm-up + 5 timed calls")
+        cur.cpu = lambda x=x: ((x.size * 4.0 + x.shape[0] * 4.0) / (orc.time_rowsum_f32(x, 5, 200) * 1e6), CPU_PROTOCOL % (5, 200))
         wl.append(cur)
 
     if want("transpose_f32"):
@@ -198,7 +203,7 @@ def build_workloads(host, orc, stream, only):
                        "f32", "transpose f32 [4096,4096] random non-NaN bits seed 20245")
         x = gen_bits(rows * cols, "f32", 20245).reshape(rows, cols)
         cur.args = [dev(x), out(rows * cols * 4), rows, cols]
-        cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_transpose2d(x, 1, 5) * 1e6), "full tensor, 1 warm-up + 5 timed calls")
+        cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_transpose2d(x, 5, 100) * 1e6), CPU_PROTOCOL % (5, 100))
         wl.append(cur)
 
     if want("transpose_bf16"):
@@ -207,7 +212,8 @@ def build_workloads(host, orc, stream, only):
                        "bf16", "transpose bf16 [8192,8192] random non-NaN bits seed 20244")
         x = gen_bits(rows * cols, "bf16", 20244).reshape(rows, cols)
         cur.args = [dev(x), out(rows * cols * 2), rows, cols]
-        cur.cpu = lambda x=x: (2.0 * x.size * 2 / (orc.time_transpose2d(x, 1, 3) * 1e6), "full tensor, 1 warm-up + 3 timed calls")
+        cur.cpu = lambda x=x: (2.0 * x.size * 2 / (orc.time_transpose2d(x, 5, 20) * 1e6),
+                             CPU_PROTOCOL % (5, 20) + " (20 instead of the template's 100: a call takes ~0.8 s)")
         wl.append(cur)
 
     if want("silu_f32"):
@@ -216,7 +222,8 @@ def build_workloads(host, orc, stream, only):
                        "silu f32 512x640x20x15 uniform(-8,8) seed 20251")
         x = gen_uniform(n, "f32", 20251, -8.0, 8.0)
         cur.args = [dev(x), out(n * 4), n]
-        cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_silu_f32(x, 0, 2) * 1e6), "full tensor, 2 timed calls")
+        cur.cpu = lambda x=x: (2.0 * x.size * 4 / (orc.time_silu_f32(x, 5, 20) * 1e6),
+                             CPU_PROTOCOL % (5, 20) + " (20 instead of the template's 100: a call takes ~0.9 s)")
         wl.append(cur)
     return wl
 
@@ -247,7 +254,9 @@ def roofline(w, ms):
     else:
         achieved, peak, unit = w.work / (ms * 1e6), HBM_PEAK_GBS, "GB/s"
     return {"bound": w.bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 4), "traffic": TRAFFIC.get(w.name)}
+            "frac": round(achieved / peak, 4), "traffic": TRAFFIC.get(w.name),
+            "traffic_source": "profiles/hbm_traffic_fetch_write_pmc.txt (rocprofv3 FETCH_SIZE / WRITE_SIZE, not measured in this run)"
+            if w.name in TRAFFIC else None}
 
 
 def measure_secondary(stream, w, rounds):
@@ -298,9 +307,6 @@ def measure_rotating(host, stream, w, passes):
     ms = stream.elapsed_ms(ev0, ev1) / (passes * copies)
     for p in extra:
         stream.free(p)
-    # A hot loop started right after these ~2 GiB are freed measures 6-10 % low, whichever workload
-    # it belongs to (the two transposes showed it on each other); a pause removes most of that.
-    time.sleep(1.5)
     return ms, copies
 
 
@@ -391,31 +397,54 @@ def main():
     stream.free(d_probe)
     log("gpuMemCopy host->device: %.1f GB/s" % h2d_gbs)
 
-    # The secondary workloads run first: the device then enters the headline loop
-    # from a loaded state.  Coming from idle, the first ~100 GEMM launches run
-    # ~10% slower while the power controller settles, which a short timed region
-    # would mostly measure.
+    # A streaming kernel on `host_shared` allocations (gpuMemAlloc with isShared: pinned host memory the
+    # GPU reads and writes over the host link): the rate a pipeline gets when it leaves its tensors in
+    # the buffers IMEX's insert-gpu-allocs pass marks host_shared instead of copying them to the device.
+    n_sh = 4096 * 4096
+    sh_in, sh_out = stream.alloc(n_sh * 4, shared=True), stream.alloc(n_sh * 4, shared=True)
+    sh_ms = stream.profile("imex_relu_f32", [n_sh], [sh_in, sh_out, n_sh], warmups=1, rounds=3, mode=1)[0] / 3
+    shared_gbs = 2.0 * n_sh * 4 / (sh_ms * 1e6)
+    stream.free(sh_in)
+    stream.free(sh_out)
+    log("imex_relu_f32 on host_shared buffers: %.1f GB/s" % shared_gbs)
+
+    # The secondary workloads run first.  Coming from idle or from lighter work, the first ~100 GEMM
+    # launches run ~10% slower while the power controller settles, which a short timed region would
+    # mostly measure: the headline loop below therefore starts with SETTLE_LAUNCHES untimed launches,
+    # whatever --warmup says.
     per = []
     secondary = sorted(workloads[1:], key=lambda w: w.bound == "mfma")  # the other GEMM goes last
     for w in secondary:
         hot_ms, cold_ms = measure_secondary(stream, w, rounds=50 if w.bound == "mfma" else 200)
         rot_ms, copies = measure_rotating(host, stream, w, passes=max(2, 200 // 24))
-        rf = roofline(w, hot_ms)
+        if w is not secondary[-1]:
+            # A hot loop started right after the ring's ~2 GiB are freed measures 6-10 % low, whichever
+            # workload it belongs to; a pause removes most of that.  Not after the last one: the headline
+            # kernel follows with its own settle phase and must not find the device idle.
+            time.sleep(1.5)
+        # `roofline` is the rotating figure: every launch streams its tensors from HBM.  Back-to-back launches
+        # on one buffer pair are served in part by the 256 MiB Infinity Cache (`roofline_cache_resident`, not an
+        # HBM fraction); `roofline_cache_flushed` is the reference profiler's protocol, which also times an
+        # event pair per launch and the write-back of the flush's dirty lines.
+        rf = roofline(w, rot_ms)
         entry_ = {"name": w.name, "workload": w.describe, "kernel": w.kernel, "dtype": w.dtype,
-                  "ms_per_launch": round(hot_ms, 5), "ms_per_launch_cache_flushed": round(cold_ms, 5),
-                  "ms_per_launch_rotating": round(rot_ms, 5), "rotating_buffer_sets": copies,
-                  "roofline": rf, "roofline_cache_flushed": roofline(w, cold_ms),
-                  "roofline_rotating": roofline(w, rot_ms)}
-        log("%s: %.4f ms (%.1f %s, %.1f%% of peak); rotating over %d buffer sets %.4f ms (%.1f%%); "
-            "cache-flushed %.4f ms (%.1f%%)" % (
-                w.name, hot_ms, rf["achieved"], rf["unit"], 100 * rf["frac"], copies, rot_ms,
-                100 * entry_["roofline_rotating"]["frac"], cold_ms, 100 * entry_["roofline_cache_flushed"]["frac"]))
+                  "ms_per_launch": round(rot_ms, 5), "rotating_buffer_sets": copies,
+                  "ms_per_launch_cache_resident": round(hot_ms, 5), "ms_per_launch_cache_flushed": round(cold_ms, 5),
+                  "roofline": rf, "roofline_protocol": "rotating: back-to-back launches over %d separate buffer sets (>= 2 GiB)" % copies,
+                  "roofline_cache_flushed": roofline(w, cold_ms),
+                  "roofline_cache_resident": roofline(w, hot_ms)}
+        log("%s: rotating over %d buffer sets %.4f ms (%.1f %s, %.1f%% of peak); cache-flushed %.4f ms (%.1f%%); "
+            "same buffers back to back %.4f ms (%.1f%%)" % (
+                w.name, copies, rot_ms, rf["achieved"], rf["unit"], 100 * rf["frac"], cold_ms,
+                100 * entry_["roofline_cache_flushed"]["frac"], hot_ms, 100 * entry_["roofline_cache_resident"]["frac"]))
         per.append(entry_)
 
     head = workloads[0]
     K, W = args.steps, args.warmup
     step = stream.prepare(head.kernel, head.dims, head.args)
-    for _ in range(max(W, 1)):
+    for _ in range(SETTLE_LAUNCHES):
+        step()
+    for _ in range(W):
         step()
     stream.wait()
     t0 = time.perf_counter()
@@ -428,23 +457,25 @@ def main():
     wall_ms = (t1 - t0) * 1e3 / K
     event_ms = stream.elapsed_ms(ev0, ev1) / K
     # device-side duration of a launch: back-to-back launches from C, no Python in the loop
-    kernel_ms = stream.profile(head.kernel, head.dims, head.args, warmups=3, rounds=K, mode=1)[0] / K
+    b2b = max(K, 200)
+    kernel_ms = stream.profile(head.kernel, head.dims, head.args, warmups=20, rounds=b2b, mode=1)[0] / b2b
     log("%s: wall %.4f ms/step, events %.4f ms/step, back-to-back %.4f ms/launch" % (head.name, wall_ms, event_ms, kernel_ms))
     value = head.work / (wall_ms * 1e9)
 
     # What the matrix pipe sustains on this kind of operand data with nothing else going on
-    # (imex_mfma_lds_ceiling_f16: MFMA 16x16x32 fed from LDS, no global traffic), measured right
-    # after the headline loop so the part is in the same thermal / power state.
+    # (imex_mfma_lds_ceiling_f16 in lib/imex_probe.hsaco: MFMA 16x16x32 fed from LDS, no global traffic),
+    # measured right after the headline loop so the part is in the same thermal / power state.
     ceiling = {}
     groups, iters = info["cus"], 2048
     d_sink = stream.alloc(groups * 512 * 4)
-    for label, zero in (("f16_uniform_pm1", 0), ("zeros", 1)):
-        cargs = [d_sink, groups * 512, iters, zero]
-        ms = stream.profile("imex_mfma_lds_ceiling_f16", [groups * 512], cargs, warmups=100, rounds=200, mode=1)[0] / 200
+    probe_fn = stream.kernel_from_file(host.PROBE_CODE_OBJECT, "imex_mfma_lds_ceiling_f16")
+    for label, mode in (("f16_uniform_pm1", 0), ("zeros", 1), ("f16_every_exponent", 2)):
+        ms = stream.profile_function(probe_fn, (groups, 1, 1), (512, 1, 1), [d_sink, groups * 512, iters, mode],
+                                     warmups=100, rounds=200)
         ceiling[label] = round(groups * 8.0 * iters * 32 * 16384 / (ms * 1e9), 1)
     stream.free(d_sink)
-    log("MFMA-from-LDS ceiling: %.0f TFLOP/s on f16 in (-1,1), %.0f TFLOP/s on zeros" % (
-        ceiling["f16_uniform_pm1"], ceiling["zeros"]))
+    log("MFMA-from-LDS ceiling: %.0f TFLOP/s on f16 uniform in (-1,1), %.0f on zeros, %.0f with every exponent equally likely" % (
+        ceiling["f16_uniform_pm1"], ceiling["zeros"], ceiling["f16_every_exponent"]))
 
     result = {
         "metric": METRIC, "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -453,12 +484,15 @@ def main():
         "config": {"workload": "BASELINE.json configs[3]: " + head.describe, "kernel": head.kernel,
                    "launch": "grid (256,1,1) x block (512,1,1)", "device": info["name"],
                    "cus": info["cus"], "clock_mhz": info["clock_khz"] / 1e3,
-                   "gpuMemCopy_h2d_GBps": round(h2d_gbs, 1)},
+                   "gpuMemCopy_h2d_GBps": round(h2d_gbs, 1),
+                   "relu_f32_on_host_shared_buffers_GBps": round(shared_gbs, 1)},
         # `achieved` prices the launch at its HIP-event duration over the timed region
         "roofline": dict(roofline(head, event_ms), event_ms_per_step=round(event_ms, 5),
                          back_to_back_ms=round(kernel_ms, 5)),
+        "settle_launches": SETTLE_LAUNCHES,
         # context for `roofline`, not a replacement for its published peak: TFLOP/s of a loop of
-        # nothing but MFMA 16x16x32 + LDS operand reads on hashed f16 in (-1,1) and on zeros
+        # nothing but MFMA 16x16x32 + LDS operand reads on f16 uniform in (-1,1), on zeros, and on
+        # f16 with random mantissas and every exponent below 1.0 equally likely
         "mfma_lds_ceiling_tflops": ceiling,
     }
 

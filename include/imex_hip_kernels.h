@@ -56,10 +56,6 @@
  *   imex_gemm_4kx4kx4k_transpose_a       (At, B, C)       dims = {}   C += A^T.B
  *       the reference kernels' own signatures (WG/...f32.mlir:48, ...bias.mlir:78,
  *       ...transpose_b.mlir:53, ...transpose_a.mlir:31)
- *   imex_mfma_lds_ceiling_f16      (out:f32*, outCount:i64, iters:i64, zero:i64)   dims = {outCount}
- *       a measurement kernel with no counterpart in the reference: `iters` steps of 32 MFMA
- *       16x16x32 per wavefront on operands read from LDS (hashed f16 in (-1,1), or zeros),
- *       no global traffic; gridX * 8 * iters * 32 * 16384 FLOP; one f32 per lane stored below outCount
  */
 #ifndef IMEX_HIP_KERNELS_H
 #define IMEX_HIP_KERNELS_H

@@ -102,6 +102,15 @@ void gpuWait(void *queue);
  * reference wrapper; modules live for the process, so this is a no-op. */
 void gpuModuleUnload(void *queue, void *module);
 
+/* `count` 32-bit (16-bit) elements at `dst` set to `value`, asynchronously on the stream; gpuWait or a
+ * later launch on the stream orders after it.  No reference line to cite: `gpux.memset` exists as an
+ * op but convert-gpux-to-llvm has no pattern for it (lib/Conversion/GPUXToLLVM/GPUXToLLVMPass.cpp:828-840
+ * lists the lowered ops), so these two names and signatures are this library's -- the stream-first
+ * form of the upstream callees below, for a lowering to bind when one is added.  `dst` must be
+ * aligned to the element size.  Runs as a kernel of this library, never as a memset on the stream. */
+void gpuMemSet32(void *queue, void *dst, unsigned int value, size_t count);
+void gpuMemSet16(void *queue, void *dst, unsigned short value, size_t count);
+
 /* ---- upstream gpu-to-llvm ABI (LevelZeroRuntimeWrappers.cpp:673-741) ---- */
 void *mgpuStreamCreate(void);
 void mgpuStreamSynchronize(void *stream);
@@ -115,6 +124,9 @@ void mgpuMemcpy(void *dst, void *src, size_t bytes, void *stream);
 /* `count` 32-bit words of `value`.  Runs as a kernel of this library (not as a memset on the stream), so a
  * caller that captures the stream into a HIP graph gets an ordinary kernel node. */
 void mgpuMemset32(void *dst, unsigned int value, size_t count, void *stream);
+/* The 16-bit callee of the upstream gpu.memset lowering (f16 / bf16 / i16 fills); the reference
+ * wrapper exports only the 32-bit one (LevelZeroRuntimeWrappers.cpp:705-711). */
+void mgpuMemset16(void *dst, unsigned short value, size_t count, void *stream);
 void *mgpuModuleLoad(const void *data, size_t dataSize);
 void *mgpuModuleGetFunction(void *module, const char *name);
 void mgpuModuleUnload(void *module);
@@ -135,12 +147,13 @@ int imexHipProfileKernel(void *queue, void *kernel, size_t gridX, size_t gridY, 
                          void *params, int warmups, int rounds, size_t flushBytes, int mode,
                          float *times_ms);
 
-/* Records a timestamp event at the stream's current tail (owned by the stream). */
+/* Records a timestamp event at the stream's current tail (owned by the stream; the handle is good
+ * until 1024 further timestamps have been recorded on that stream). */
 void *imexHipRecordTimestamp(void *queue);
 
-/* Milliseconds between two events of one stream.  Use imexHipRecordTimestamp
- * events for timing: an event returned by gpuLaunchKernel is an ordering point,
- * whose timestamp is taken when it is first used. */
+/* Milliseconds between two imexHipRecordTimestamp events of one stream.  An event returned by
+ * gpuLaunchKernel is refused (error convention above): it is an ordering point whose HIP event
+ * is only recorded when it is first waited on, so it carries no time of its own. */
 float imexHipEventElapsedMs(void *startEvent, void *stopEvent);
 
 /* out[9] = avg, min, max, median, stddev, variance, P95, P5, middle-third avg

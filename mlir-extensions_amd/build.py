@@ -4,6 +4,7 @@ Everything is compiled in-tree with explicit ``hipcc`` / ``gcc`` command lines
 (no CMake needed, hipcc cross-compiles gfx950 without a GPU present):
 
   lib/imex_<group>.hsaco        one code object per kernel source file
+  lib/imex_probe.hsaco          measurement kernels (bench.py and the driver load the file; not in the catalogue)
   lib/libimex-hip-kernels.so    catalogue + the code objects embedded as blobs
   lib/libimex-hip-runtime.so    the gpu* / mgpu* runtime-wrapper ABI on HIP
   lib/libimex_runner_utils.so   _mlir_ciface_* host helpers
@@ -27,7 +28,10 @@ INCLUDE_DIR = os.path.join(REPO_DIR, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
-KERNEL_GROUPS = ["eltwise", "softmax", "reduce", "transpose", "gemm", "fusion", "attention", "probe"]
+KERNEL_GROUPS = ["eltwise", "softmax", "reduce", "transpose", "gemm", "fusion", "attention"]
+# Measurement kernels: a code object of their own (lib/imex_probe.hsaco) that bench.py and the
+# driver load from the file; the catalogue library holds operators only.
+BENCH_ONLY_GROUPS = ["probe"]
 
 # -ffp-contract=off: the SiLU, scalar-GEMM and reduction kernels rely on
 # separately rounded multiplies and adds.  Packed-FP32 instruction selection is
@@ -54,7 +58,7 @@ def _run(cmd, verbose):
 
 def build_kernels(verbose=False, groups=None):
     os.makedirs(LIB_DIR, exist_ok=True)
-    for g in groups or KERNEL_GROUPS:
+    for g in groups or KERNEL_GROUPS + BENCH_ONLY_GROUPS:
         src = os.path.join(CSRC, "kernels", g + ".hip")
         out = os.path.join(LIB_DIR, "imex_%s.hsaco" % g)
         _run([HIPCC] + DEVICE_FLAGS + [src, "-o", out], verbose)

@@ -40,6 +40,8 @@
 #include <string>
 #include <vector>
 
+#include <unistd.h>
+
 namespace {
 
 enum class Elem { F32, F16, BF16 };
@@ -61,6 +63,7 @@ struct Workload {
   int floatArg;                 // 0 none; 1 trailing f32 `init` (reductions); 2 f32 between pointers and indices (sm_scale)
   double work;                  // algorithmic bytes or flops per launch
   bool mfma;                    // roofline: MFMA (TFLOP/s) or HBM (GB/s)
+  bool probe = false;           // a measurement kernel: loaded from imex_probe.hsaco beside this program, one lane per dims[0]
 };
 
 std::vector<Workload> workloads() {
@@ -87,6 +90,12 @@ std::vector<Workload> workloads() {
       {"gemm_f16_4096", "imex_gemm_f16_f16_f32", {K4, K4, K4},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true},
+      // the reference's bias kernel with its own argument order (bias, C, A, B): C = bias[n] + (C + A.B)
+      // (WG/gemm_4kx4kx4k_f16_f16_f32_bias.mlir:77-116); C is input and output
+      {"gemm_f16_4096_bias", "imex_gemm_4kx4kx4k_f16_f16_f32_bias", {},
+       {{Elem::F32, {K4}, true, -1, 1}, {Elem::F32, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -0.5f, 0.5f},
+        {Elem::F16, {K4, K4}, true, -0.5f, 0.5f}},
+       {}, 0, 2.0 * K4 * K4 * K4, true},
       {"gemm_f16_4096_f16_out", "imex_gemm_f16_f16_f16", {K4, K4, K4},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true},
@@ -149,12 +158,15 @@ std::vector<Workload> workloads() {
       {"input_fusion_f32_8192x8192", "imex_input_fusion_f32", {K8, K8},
        {{Elem::F32, {K8, K8}, true, -3, 3}, {Elem::F32, {K8, K8}, true, 0.5f, 3}, {Elem::F32, {K8}, false, 0, 0}},
        {K8, K8}, 0, 2.0 * K8 * K8 * 4 + K8 * 4, false},
-      // not operators: the MFMA pipe fed from LDS with nothing else going on, one workgroup per CU,
-      // on hashed f16 operands in (-1,1) and on zeros -- the rate the GEMMs' operand values allow
-      {"mfma_lds_ceiling_f16_random", "imex_mfma_lds_ceiling_f16", {256 * 512},
-       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 0}, 0, 256.0 * 8 * 2048 * 32 * 16384, true},
+      // not operators (and not in the catalogue): the MFMA pipe fed from LDS with nothing else going on, one
+      // workgroup per CU, on f16 operands uniform in (-1,1) like the GEMM benchmark's, on zeros, and on f16 with
+      // every exponent equally likely -- the rate the operand values allow
+      {"mfma_lds_ceiling_f16_uniform", "imex_mfma_lds_ceiling_f16", {256 * 512},
+       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 0}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
       {"mfma_lds_ceiling_f16_zeros", "imex_mfma_lds_ceiling_f16", {256 * 512},
-       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 1}, 0, 256.0 * 8 * 2048 * 32 * 16384, true},
+       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 1}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
+      {"mfma_lds_ceiling_f16_every_exponent", "imex_mfma_lds_ceiling_f16", {256 * 512},
+       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 2}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
   };
 }
 
@@ -179,6 +191,18 @@ void fillHost(void *host, const Tensor &t) {
   }
 }
 
+// Directory of this executable (the code objects that are not in the catalogue sit beside it).
+std::string programDir() {
+  char buf[4096];
+  const ssize_t n = readlink("/proc/self/exe", buf, sizeof buf - 1);
+  if (n <= 0)
+    return ".";
+  buf[n] = 0;
+  std::string p(buf);
+  const size_t slash = p.rfind('/');
+  return slash == std::string::npos ? "." : p.substr(0, slash);
+}
+
 struct Options {
   int runs = 100, warmups = 10, launchOnly = 0;
   bool flush = false, zeros = false;
@@ -199,13 +223,33 @@ int runWorkload(const Workload &w, const Options &opt) {
     }
   }
 
-  size_t grid[3], block[3], smem = 0;
-  if (imexHipKernelLaunchShape(w.kernel, w.dims.data(), static_cast<int>(w.dims.size()), grid, block, &smem) != 0) {
-    fprintf(stderr, "%s: no launch shape for %s\n", w.name, w.kernel);
-    return 1;
-  }
+  size_t grid[3] = {1, 1, 1}, block[3] = {512, 1, 1}, smem = 0;
   size_t blobSize = 0;
-  const void *blob = imexHipKernelModule(w.kernel, &blobSize);
+  const void *blob = nullptr;
+  static std::vector<char> probeBlob; // kept for the life of the process: the runtime caches modules by address
+  if (w.probe) {
+    grid[0] = static_cast<size_t>((w.dims[0] + 511) / 512);
+    if (probeBlob.empty()) {
+      const std::string path = programDir() + "/imex_probe.hsaco";
+      FILE *f = fopen(path.c_str(), "rb");
+      if (!f) {
+        fprintf(stderr, "%s: cannot read %s\n", w.name, path.c_str());
+        return 1;
+      }
+      char buf[65536];
+      for (size_t n; (n = fread(buf, 1, sizeof buf, f)) > 0;)
+        probeBlob.insert(probeBlob.end(), buf, buf + n);
+      fclose(f);
+    }
+    blob = probeBlob.data();
+    blobSize = probeBlob.size();
+  } else {
+    if (imexHipKernelLaunchShape(w.kernel, w.dims.data(), static_cast<int>(w.dims.size()), grid, block, &smem) != 0) {
+      fprintf(stderr, "%s: no launch shape for %s\n", w.name, w.kernel);
+      return 1;
+    }
+    blob = imexHipKernelModule(w.kernel, &blobSize);
+  }
   void *module = gpuModuleLoad(stream, blob, blobSize);
   void *kernel = gpuKernelGet(stream, module, w.kernel);
 

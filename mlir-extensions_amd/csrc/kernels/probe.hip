@@ -13,15 +13,21 @@
 // benchmark uses, so the GEMM's rate can be held against what the silicon
 // sustains on that data as well as against the published peak.
 //
-//   imex_mfma_lds_ceiling_f16(out: f32*, outCount: i64, iters: i64, zero: i64)
+//   imex_mfma_lds_ceiling_f16(out: f32*, outCount: i64, iters: i64, mode: i64)
 //
 // Each workgroup (512 lanes = 8 wavefronts, two per SIMD, like the GEMM) fills
-// 64 KiB of LDS with hashed f16 pairs in (-1, 1) -- or zeros if `zero` != 0 --
-// and then runs `iters` steps of the GEMM's K-step: 8 A fragments + 4 B fragments
+// 64 KiB of LDS with hashed f16 pairs and then runs `iters` steps of the GEMM's K-step: 8 A fragments + 4 B fragments
 // read from LDS with ds_read_b128 at a position that moves every step, 32 MFMA
 // 16x16x32 on them (a 128 x 64 x 32 product per wavefront).  FLOP per launch =
 // gridX * 8 * iters * 32 * 2*16*16*32.  One f32 per lane is stored at the end
 // (guarded by outCount) so the work is observable.
+//
+// mode 0: values uniform in (-1, 1) rounded to f16, the distribution of the GEMM
+//         benchmark's operands (half of them have the exponent of 0.5, a quarter
+//         the one below, ...);
+// mode 1: zeros;
+// mode 2: random sign and mantissa with every exponent below 1.0 equally likely --
+//         more bits switching per operand than mode 0, and a lower sustained rate.
 //
 // The MFMA shape matters for this ceiling: on the same random operands a loop of
 // 32x32x16 instructions with the same LDS bytes per FLOP sustained about 9 % less
@@ -44,17 +50,22 @@ constexpr int kFragsA = 8, kFragsB = 4;
 } // namespace
 
 extern "C" __global__ __launch_bounds__(kThreads) void imex_mfma_lds_ceiling_f16(float *out, int64_t outCount,
-                                                                                  int64_t iters, int64_t zero) {
+                                                                                  int64_t iters, int64_t mode) {
   __shared__ __attribute__((aligned(16))) uint32_t lds[kLdsBytes / 4];
   for (int i = threadIdx.x; i < kLdsBytes / 4; i += kThreads) {
     uint32_t x = (static_cast<uint32_t>(i) + blockIdx.x * 7919u) * 2654435761u;
     x ^= x >> 15;
     x *= 2246822519u;
     x ^= x >> 13;
-    // two f16 values: random sign and mantissa, exponent field 0..14, i.e. |v| < 1
-    const uint32_t lo = (x & 0x83ffu) | (((x >> 10) % 15u) << 10);
-    const uint32_t hi = ((x >> 16) & 0x83ffu) | (((x >> 26) % 15u) << 10);
-    lds[i] = zero ? 0u : (lo | (hi << 16));
+    uint32_t lo, hi;
+    if (mode == 2) { // random sign and mantissa, exponent field 0..14, i.e. |v| < 1
+      lo = (x & 0x83ffu) | (((x >> 10) % 15u) << 10);
+      hi = ((x >> 16) & 0x83ffu) | (((x >> 26) % 15u) << 10);
+    } else {         // h / 32768 - 1 for each 16-bit half h: uniform in [-1, 1), exact in f32, one rounding to f16
+      lo = imexhip::float_to_half_bits(static_cast<float>(x & 0xffffu) * (1.0f / 32768.0f) - 1.0f);
+      hi = imexhip::float_to_half_bits(static_cast<float>(x >> 16) * (1.0f / 32768.0f) - 1.0f);
+    }
+    lds[i] = mode == 1 ? 0u : (lo | (hi << 16));
   }
   __syncthreads();
 

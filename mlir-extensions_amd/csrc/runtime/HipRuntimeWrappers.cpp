@@ -78,6 +78,7 @@ struct LaunchEvent {
   uint64_t sequence;    // the launch this slot currently stands for
   hipEvent_t event;     // null until someone waits on or times a position of this slot
   uint64_t recordedFor; // sequence `event` was last recorded for (0: never)
+  bool isTimestamp;     // recorded when it was handed out (imexHipRecordTimestamp), so it marks a point in time
 };
 
 // Launch events live in a ring: a handle stays valid for the life of its stream,
@@ -85,6 +86,9 @@ struct LaunchEvent {
 // same in-order stream -- waiting on a stale handle over-synchronises, it never
 // under-synchronises -- so a process that launches for days does not grow.
 constexpr size_t kEventSlots = 4096;
+// Timestamps come from a ring of their own: a handle is good until kTimestampSlots further
+// timestamps have been recorded on its stream, then its slot is recorded anew.
+constexpr size_t kTimestampSlots = 1024;
 
 struct GpuHipQueue {
   int device = 0;
@@ -92,7 +96,8 @@ struct GpuHipQueue {
   bool ownsStream = true;
   uint64_t launches = 0;
   std::vector<LaunchEvent> ring;          // handed out by gpuLaunchKernel, slot = launch number mod ring size
-  std::vector<LaunchEvent *> timestamps;  // handed out by imexHipRecordTimestamp; kept until the stream goes
+  std::vector<LaunchEvent> timestamps;    // handed out by imexHipRecordTimestamp, slot = timestamp number mod ring size
+  uint64_t timestampCount = 0;
   void *flushBuffer = nullptr;    // scratch for the profiler's cache flush
   size_t flushBytes = 0;
 
@@ -107,23 +112,42 @@ struct GpuHipQueue {
     }
   }
 
-  ~GpuHipQueue() noexcept(false) {
+  // Waits for the stream and releases what the queue owns; throws on a HIP error (the callers
+  // run it under catchAll before deleting the queue).  Idempotent.
+  void release() {
+    if (!stream)
+      return;
     CHECK_HIP(hipSetDevice(device));
     CHECK_HIP(hipStreamSynchronize(stream));
-    for (LaunchEvent &e : ring)
-      if (e.event)
-        CHECK_HIP(hipEventDestroy(e.event));
-    for (LaunchEvent *e : timestamps) {
-      if (e->event)
-        CHECK_HIP(hipEventDestroy(e->event));
-      delete e;
+    for (std::vector<LaunchEvent> *events : {&ring, &timestamps}) {
+      for (LaunchEvent &e : *events)
+        if (e.event)
+          CHECK_HIP(hipEventDestroy(e.event));
+      events->clear();
     }
     if (flushBuffer)
       CHECK_HIP(hipFree(flushBuffer));
+    flushBuffer = nullptr;
     if (ownsStream)
       CHECK_HIP(hipStreamDestroy(stream));
+    stream = nullptr;
+  }
+
+  // A queue that was not released (a thread's default queue at thread exit): best effort, no throw.
+  ~GpuHipQueue() {
+    try {
+      release();
+    } catch (...) {
+    }
   }
 };
+
+void destroyQueue(GpuHipQueue *queue) {
+  if (!queue)
+    return;
+  queue->release();
+  delete queue;
+}
 
 int defaultDeviceOrdinal() {
   if (const char *env = getenv("IMEX_HIP_DEVICE"))
@@ -395,10 +419,12 @@ void profile(GpuHipQueue *queue, LaunchArgs &la, int warmups, int rounds, size_t
   CHECK_HIP(hipEventDestroy(stop));
 }
 
-long envLong(const char *name, long fallback) {
+// An integer environment variable; anything unparsable or below `least` gives the fallback.
+long envLong(const char *name, long fallback, long least = 1) {
   if (const char *v = getenv(name)) {
-    long parsed = strtol(v, nullptr, 10);
-    if (parsed > 0)
+    char *end = nullptr;
+    long parsed = strtol(v, &end, 10);
+    if (end != v && parsed >= least)
       return parsed;
   }
   return fallback;
@@ -437,7 +463,7 @@ LaunchEvent *launchKernel(GpuHipQueue *queue, void *kernel, size_t gx, size_t gy
     // Defaults of LevelZeroRuntimeWrappers.cpp:521-523; a positive
     // IMEX_PROFILING_RUNS / IMEX_PROFILING_WARMUPS overrides them.
     const int rounds = static_cast<int>(envLong("IMEX_PROFILING_RUNS", 1000));
-    const int warmups = static_cast<int>(envLong("IMEX_PROFILING_WARMUPS", 3));
+    const int warmups = static_cast<int>(envLong("IMEX_PROFILING_WARMUPS", 3, /*least=*/0)); // 0 = no warm-up (:547-551)
     size_t flushBytes = 0;
     if (getenv("IMEX_ENABLE_CACHE_FLUSHING"))
       flushBytes = static_cast<size_t>(envLong("IMEX_CACHE_FLUSH_BYTES", 512l << 20));
@@ -457,7 +483,7 @@ LaunchEvent *launchKernel(GpuHipQueue *queue, void *kernel, size_t gx, size_t gy
 
   enqueue(queue, la);
   if (queue->ring.empty())
-    queue->ring.assign(kEventSlots, LaunchEvent{queue, 0, nullptr, 0});
+    queue->ring.assign(kEventSlots, LaunchEvent{queue, 0, nullptr, 0, false});
   LaunchEvent *done = &queue->ring[queue->launches % kEventSlots];
   done->sequence = ++queue->launches; // a HIP event left from the slot's previous life is re-recorded on first use
   return done;
@@ -466,10 +492,41 @@ LaunchEvent *launchKernel(GpuHipQueue *queue, void *kernel, size_t gx, size_t gy
 // Default stream for the mgpu* entry points that carry no stream
 // (LevelZeroRuntimeWrappers.cpp:676).
 GpuHipQueue *defaultQueue() {
-  thread_local GpuHipQueue *q = nullptr;
+  struct Holder { // released when the thread ends
+    GpuHipQueue *q = nullptr;
+    ~Holder() { delete q; }
+  };
+  thread_local Holder holder;
+  if (!holder.q)
+    holder.q = new GpuHipQueue(defaultDeviceOrdinal(), nullptr);
+  return holder.q;
+}
+
+// The fill kernels this library carries (csrc/runtime/fill.hip), embedded at build time.
+extern "C" const char imex_runtime_fill_blob[], imex_runtime_fill_blob_end[];
+
+// `count` elements of `bits` (16 or 32) wide, each set to the low bits of `value`.  A kernel launch, not
+// a memset on the stream: memset nodes recorded into a captured HIP graph have replayed wrongly on this
+// platform, and the queue may sit on a stream its owner captures.
+void fillMemory(GpuHipQueue *q, void *dst, unsigned value, size_t count, int bits) {
   if (!q)
-    q = new GpuHipQueue(defaultDeviceOrdinal(), nullptr);
-  return q;
+    throw std::runtime_error("memset: null stream");
+  if (count == 0)
+    return;
+  if (!dst)
+    throw std::runtime_error("memset: null pointer with non-zero count");
+  if (reinterpret_cast<uintptr_t>(dst) % (bits / 8))
+    throw std::runtime_error("memset: destination is not aligned to its " + std::to_string(bits) + "-bit elements");
+  CHECK_HIP(hipSetDevice(q->device));
+  hipModule_t module =
+      loadModule(q, imex_runtime_fill_blob, size_t(imex_runtime_fill_blob_end - imex_runtime_fill_blob));
+  hipFunction_t fill = getKernel(module, bits == 32 ? "imex_runtime_fill_b32" : "imex_runtime_fill_b16");
+  uint32_t word = value;
+  int64_t n = static_cast<int64_t>(count);
+  void *params[] = {&dst, &word, &n};
+  const size_t perGroup = 256 * 4 * (128 / bits); // 256 lanes, about four 16-byte stores each
+  const unsigned groups = static_cast<unsigned>(std::min<size_t>((count + perGroup - 1) / perGroup, 2048));
+  CHECK_HIP(hipModuleLaunchKernel(fill, groups, 1, 1, 256, 1, 1, 0, q->stream, params, nullptr));
 }
 
 GpuHipQueue *asQueue(void *p) { return static_cast<GpuHipQueue *>(p); }
@@ -488,7 +545,7 @@ extern "C" void *gpuCreateStream(void *device, void *context) {
 }
 
 extern "C" void gpuStreamDestroy(void *queue) {
-  catchAll([&]() { delete asQueue(queue); });
+  catchAll([&]() { destroyQueue(asQueue(queue)); });
 }
 
 extern "C" void *gpuMemAlloc(void *queue, size_t size, size_t alignment, int isShared) {
@@ -533,6 +590,14 @@ extern "C" void gpuModuleUnload(void * /*queue*/, void * /*module*/) {
   // Modules are cached for the life of the process.
 }
 
+extern "C" void gpuMemSet32(void *queue, void *dst, unsigned int value, size_t count) {
+  catchAll([&]() { fillMemory(asQueue(queue), dst, value, count, 32); });
+}
+
+extern "C" void gpuMemSet16(void *queue, void *dst, unsigned short value, size_t count) {
+  catchAll([&]() { fillMemory(asQueue(queue), dst, value, count, 16); });
+}
+
 // ===========================================================================
 // Upstream gpu-to-llvm ABI
 // ===========================================================================
@@ -550,7 +615,7 @@ extern "C" void mgpuStreamSynchronize(void *stream) {
 }
 
 extern "C" void mgpuStreamDestroy(void *stream) {
-  catchAll([&]() { delete asQueue(stream); });
+  catchAll([&]() { destroyQueue(asQueue(stream)); });
 }
 
 extern "C" void mgpuLaunchKernel(void *kernel, size_t gridX, size_t gridY, size_t gridZ, size_t blockX,
@@ -585,27 +650,12 @@ extern "C" void mgpuMemcpy(void *dst, void *src, size_t bytes, void *stream) {
   catchAll([&]() { copyMemory(stream ? asQueue(stream) : defaultQueue(), dst, src, bytes); });
 }
 
-// The fill kernel this library carries (csrc/runtime/fill.hip), embedded at build time.
-extern "C" const char imex_runtime_fill_blob[], imex_runtime_fill_blob_end[];
-
-// A kernel launch, not a memset on the stream: memset nodes recorded into a captured HIP graph
-// have replayed wrongly on this platform, and the queue may sit on a stream its owner captures.
 extern "C" void mgpuMemset32(void *dst, unsigned int value, size_t count, void *stream) {
-  catchAll([&]() {
-    GpuHipQueue *q = stream ? asQueue(stream) : defaultQueue();
-    if (count == 0)
-      return;
-    CHECK_HIP(hipSetDevice(q->device));
-    hipModule_t module =
-        loadModule(q, imex_runtime_fill_blob, size_t(imex_runtime_fill_blob_end - imex_runtime_fill_blob));
-    hipFunction_t fill = getKernel(module, "imex_runtime_fill_b32");
-    uint32_t word = value;
-    int64_t n = static_cast<int64_t>(count);
-    void *params[] = {&dst, &word, &n};
-    const size_t perGroup = 256 * 4 * 4; // 256 lanes, about four 16-byte stores each
-    const unsigned groups = static_cast<unsigned>(std::min<size_t>((count + perGroup - 1) / perGroup, 2048));
-    CHECK_HIP(hipModuleLaunchKernel(fill, groups, 1, 1, 256, 1, 1, 0, q->stream, params, nullptr));
-  });
+  catchAll([&]() { fillMemory(stream ? asQueue(stream) : defaultQueue(), dst, value, count, 32); });
+}
+
+extern "C" void mgpuMemset16(void *dst, unsigned short value, size_t count, void *stream) {
+  catchAll([&]() { fillMemory(stream ? asQueue(stream) : defaultQueue(), dst, value, count, 16); });
 }
 
 extern "C" void *mgpuModuleLoad(const void *data, size_t dataSize) {
@@ -645,8 +695,10 @@ extern "C" void *imexHipRecordTimestamp(void *queue) {
     if (!queue)
       throw std::runtime_error("imexHipRecordTimestamp: null stream");
     GpuHipQueue *q = asQueue(queue);
-    LaunchEvent *le = new LaunchEvent{q, q->launches + 1, nullptr, 0};
-    q->timestamps.push_back(le);
+    if (q->timestamps.empty())
+      q->timestamps.assign(kTimestampSlots, LaunchEvent{q, 0, nullptr, 0, true});
+    LaunchEvent *le = &q->timestamps[q->timestampCount % kTimestampSlots];
+    le->sequence = ++q->timestampCount; // differs from what the slot was last recorded for: recorded anew, now
     materialise(le);
     return le;
   });
@@ -656,8 +708,13 @@ extern "C" float imexHipEventElapsedMs(void *startEvent, void *stopEvent) {
   return catchAll([&]() {
     if (!startEvent || !stopEvent)
       throw std::runtime_error("imexHipEventElapsedMs: null event");
-    hipEvent_t a = materialise(static_cast<LaunchEvent *>(startEvent));
-    hipEvent_t b = materialise(static_cast<LaunchEvent *>(stopEvent));
+    LaunchEvent *first = static_cast<LaunchEvent *>(startEvent), *second = static_cast<LaunchEvent *>(stopEvent);
+    // An event returned by gpuLaunchKernel is an ordering point whose HIP event is only recorded when
+    // somebody first waits on it: it carries no time of its own.
+    if (!first->isTimestamp || !second->isTimestamp)
+      throw std::runtime_error("imexHipEventElapsedMs: both events must come from imexHipRecordTimestamp");
+    hipEvent_t a = materialise(first);
+    hipEvent_t b = materialise(second);
     float ms = 0.0f;
     CHECK_HIP(hipEventSynchronize(b));
     CHECK_HIP(hipEventElapsedTime(&ms, a, b));

@@ -22,13 +22,12 @@ extern const unsigned char imex_blob_transpose[], imex_blob_transpose_end[];
 extern const unsigned char imex_blob_gemm[], imex_blob_gemm_end[];
 extern const unsigned char imex_blob_fusion[], imex_blob_fusion_end[];
 extern const unsigned char imex_blob_attention[], imex_blob_attention_end[];
-extern const unsigned char imex_blob_probe[], imex_blob_probe_end[];
 }
 
 namespace {
 
-enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm, Fusion, Attention, Probe };
-enum class Shape { Eltwise32, Eltwise16, Fusion32, Fusion16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, ReduceOuter16, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, Attention, LanesOf512 };
+enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm, Fusion, Attention };
+enum class Shape { Eltwise32, Eltwise16, Fusion32, Fusion16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, ReduceOuter16, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, Attention };
 
 struct Entry {
   const char *name;
@@ -93,9 +92,6 @@ const Entry kEntries[] = {
     {"imex_gemm_4kx4kx4k_transpose_a", "(At: f16* [K,M], B: f16*, C: f32*)", Module::Gemm, Shape::GemmFixed4k, 0},
     {"imex_gemm_4kx4kx4k_f16_f16_f32_bias", "(bias: f32*, C: f32*, A: f16*, B: f16*)", Module::Gemm,
      Shape::GemmFixed4k, 0},
-    // measurement kernel, not an operator: the MFMA pipe fed from LDS, nothing else
-    {"imex_mfma_lds_ceiling_f16", "(out: f32*, outCount: i64, iters: i64, zero: i64)", Module::Probe,
-     Shape::LanesOf512, 1},
 };
 constexpr int kEntryCount = sizeof(kEntries) / sizeof(kEntries[0]);
 
@@ -135,7 +131,6 @@ extern "C" const void *imexHipKernelModule(const char *kernel, size_t *size) {
   case Module::Gemm: begin = imex_blob_gemm; end = imex_blob_gemm_end; break;
   case Module::Fusion: begin = imex_blob_fusion; end = imex_blob_fusion_end; break;
   case Module::Attention: begin = imex_blob_attention; end = imex_blob_attention_end; break;
-  case Module::Probe: begin = imex_blob_probe; end = imex_blob_probe_end; break;
   }
   if (size)
     *size = static_cast<size_t>(end - begin);
@@ -259,10 +254,6 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     grid[0] = tileable ? ceilDiv(M, 256) * ceilDiv(N, 256) : ceilDiv(M * N, 512);
     break;
   }
-  case Shape::LanesOf512: // dims = {outCount}: one lane per output element, 512 per workgroup
-    block[0] = 512;
-    grid[0] = ceilDiv(dims[0], 512);
-    break;
   case Shape::GemmFixed4k: // the reference's own launch: blocks (16,16,1), threads (512,1,1)
     block[0] = 512;
     grid[0] = 16;

@@ -1,8 +1,9 @@
-// The runtime library's own device code: a 32-bit pattern fill.
+// The runtime library's own device code: 32-bit and 16-bit pattern fills.
 //
-// mgpuMemset32 (lib/ExecutionEngine/LEVELZERORUNTIME/LevelZeroRuntimeWrappers.cpp:705-711, the
-// upstream gpu.memset lowering) runs this kernel instead of recording a memset on the stream,
-// so that a caller who captures the stream into a HIP graph gets an ordinary kernel node.
+// mgpuMemset32 / mgpuMemset16 (the upstream gpu.memset lowering's callees; the 32-bit one is at
+// lib/ExecutionEngine/LEVELZERORUNTIME/LevelZeroRuntimeWrappers.cpp:705-711) and gpuMemSet32 /
+// gpuMemSet16 run these kernels instead of recording a memset on the stream, so that a caller
+// who captures the stream into a HIP graph gets an ordinary kernel node.
 //
 // Launch: block (256,1,1), any grid (workgroups stride over the buffer).
 
@@ -24,4 +25,23 @@ extern "C" __global__ __launch_bounds__(256) void imex_runtime_fill_b32(uint32_t
     body[i] = v;
   for (int64_t i = head + vecs * 4 + tid; i < n; i += threads)
     dst[i] = value;
+}
+
+// 16-bit pattern: single elements up to the first 16-byte boundary, whole vectors, then the tail.
+extern "C" __global__ __launch_bounds__(256) void imex_runtime_fill_b16(uint16_t *dst, uint32_t value, int64_t n) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const int64_t tid = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t threads = int64_t(gridDim.x) * 256;
+  const uint16_t v16 = static_cast<uint16_t>(value);
+  const int64_t head = min(n, int64_t((16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15) / 2);
+  const int64_t vecs = (n - head) / 8;
+  for (int64_t i = tid; i < head; i += threads)
+    dst[i] = v16;
+  u32x4 *body = reinterpret_cast<u32x4 *>(dst + head);
+  const uint32_t w = uint32_t(v16) | (uint32_t(v16) << 16);
+  const u32x4 v = {w, w, w, w};
+  for (int64_t i = tid; i < vecs; i += threads)
+    body[i] = v;
+  for (int64_t i = head + vecs * 8 + tid; i < n; i += threads)
+    dst[i] = v16;
 }

@@ -62,6 +62,9 @@ _RUNTIME_SYMBOLS = {
     "mgpuMemFree": (None, [C.c_void_p, C.c_void_p]),
     "mgpuMemcpy": (None, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "mgpuMemset32": (None, [C.c_void_p, C.c_uint, C.c_size_t, C.c_void_p]),
+    "mgpuMemset16": (None, [C.c_void_p, C.c_ushort, C.c_size_t, C.c_void_p]),
+    "gpuMemSet32": (None, [C.c_void_p, C.c_void_p, C.c_uint, C.c_size_t]),
+    "gpuMemSet16": (None, [C.c_void_p, C.c_void_p, C.c_ushort, C.c_size_t]),
     "mgpuModuleLoad": (C.c_void_p, [C.c_void_p, C.c_size_t]),
     "mgpuModuleGetFunction": (C.c_void_p, [C.c_void_p, C.c_char_p]),
     "mgpuModuleUnload": (None, [C.c_void_p]),
@@ -101,6 +104,9 @@ def _bind(lib, table):
         fn.restype = res
         fn.argtypes = args
 
+
+_FILE_BLOBS = {}
+PROBE_CODE_OBJECT = os.path.join(LIB_DIR, "imex_probe.hsaco")
 
 _runtime = None
 _kernels = None
@@ -155,16 +161,40 @@ def launch_shape(kernel, dims):
     return tuple(grid), tuple(block), smem.value
 
 
-def _pack_params(args):
-    """ParamDesc[n+1] terminated by {NULL, 0}; keeps the value storage alive."""
+def signature_types(kernel):
+    """Argument types of a catalogue kernel, from its signature string
+    "(in: f32*, out: f32*, rows: i64, init: f32)" -> ["ptr", "ptr", "i64", "f32"]; None if unknown."""
+    k = kernels()
+    for i in range(k.imexHipKernelCount()):
+        if k.imexHipKernelName(i).decode() == kernel:
+            sig = k.imexHipKernelSignature(i).decode().strip()[1:-1]
+            types = []
+            for part in sig.split(","):
+                t = part.split(":", 1)[1].strip()
+                types.append("ptr" if "*" in t else t.split()[0])
+            return types
+    return None
+
+
+def _pack_params(args, types=None):
+    """ParamDesc[n+1] terminated by {NULL, 0}; keeps the value storage alive.  With `types` (see
+    signature_types) every scalar is packed as the kernel declares it -- a Python int given for an
+    f32 parameter becomes a 4-byte float; without, pointers are 8 bytes, ints i64 and floats f32."""
+    if types is not None and len(types) != len(args):
+        raise TypeError("kernel takes %d arguments, %d given" % (len(types), len(args)))
     storage = []
     descs = (ParamDesc * (len(args) + 1))()
     for i, a in enumerate(args):
-        if isinstance(a, Ptr):
+        want = types[i] if types is not None else None
+        if want == "ptr" or (want is None and isinstance(a, Ptr)):
+            if not isinstance(a, Ptr):
+                raise TypeError("argument %d is a memref base pointer, got %r" % (i, a))
             v = C.c_void_p(int(a))
-        elif isinstance(a, (float, np.floating)):
+        elif want == "f32" or (want is None and isinstance(a, (float, np.floating))):
             v = C.c_float(float(a))
-        elif isinstance(a, (int, np.integer)):
+        elif want == "i64" or (want is None and isinstance(a, (int, np.integer))):
+            if isinstance(a, (float, np.floating)) and float(a) != int(a):
+                raise TypeError("argument %d is an index, got %r" % (i, a))
             v = C.c_int64(int(a))
         else:
             raise TypeError("unsupported kernel argument %r" % (a,))
@@ -208,6 +238,10 @@ class Stream:
         """mgpuMemset32 on this queue: `count` 32-bit words of `value`."""
         self.rt.mgpuMemset32(int(ptr), value, count, self.handle)
 
+    def memset(self, ptr, value, count, bits=32):
+        """gpuMemSet32 / gpuMemSet16: `count` elements of `bits` width set to `value`, asynchronously."""
+        (self.rt.gpuMemSet32 if bits == 32 else self.rt.gpuMemSet16)(self.handle, int(ptr), value, count)
+
     def copy(self, dst, src, nbytes):
         self.rt.gpuMemCopy(self.handle, int(dst), int(src), nbytes)
 
@@ -231,6 +265,26 @@ class Stream:
         module = self.rt.gpuModuleLoad(self.handle, blob, size.value)
         return self.rt.gpuKernelGet(self.handle, module, name.encode())
 
+    def kernel_from_file(self, path, name):
+        """A kernel of a code object that is not part of the catalogue (the measurement kernels in
+        lib/imex_probe.hsaco): the file's bytes go to gpuModuleLoad like any other blob."""
+        blob = _FILE_BLOBS.get(path)
+        if blob is None:
+            with open(path, "rb") as f:
+                data = f.read()
+            blob = _FILE_BLOBS[path] = C.create_string_buffer(data, len(data))  # kept: the runtime caches modules by address
+        module = self.rt.gpuModuleLoad(self.handle, C.cast(blob, C.c_void_p), len(blob))
+        return self.rt.gpuKernelGet(self.handle, module, name.encode())
+
+    def profile_function(self, fn, grid, block, args, warmups, rounds):
+        """ms per launch over `rounds` back-to-back launches of an already resolved kernel."""
+        descs, keep = _pack_params(args)
+        out = (C.c_float * 1)()
+        self.rt.imexHipProfileKernel(self.handle, fn, grid[0], grid[1], grid[2], block[0], block[1], block[2], 0,
+                                     C.cast(descs, C.c_void_p), warmups, rounds, 0, 1, out)
+        del keep
+        return out[0] / rounds
+
     def launch(self, name, dims, args, deps=None, grid=None, block=None):
         """gpuModuleLoad + gpuKernelGet + gpuLaunchKernel; returns the event (or
         None when the launch shape is empty).  `grid` / `block` replace the catalogue's."""
@@ -240,7 +294,7 @@ class Stream:
         if 0 in grid:
             return None
         fn = self.kernel(name)
-        descs, keep = _pack_params(args)
+        descs, keep = _pack_params(args, signature_types(name))
         evs = (EventDesc * (len(deps or []) + 1))()
         for i, e in enumerate(deps or []):
             evs[i].event = e
@@ -257,7 +311,7 @@ class Stream:
         if 0 in grid:
             return lambda: None
         fn = self.kernel(name)
-        descs, keep = _pack_params(args)
+        descs, keep = _pack_params(args, signature_types(name))
         params = C.cast(descs, C.c_void_p)
         launch, handle = self.rt.gpuLaunchKernel, self.handle
         gx, gy, gz = grid
@@ -271,7 +325,7 @@ class Stream:
         """Per-launch times in ms (mode 0) or [total ms] over `rounds` back-to-back launches (mode 1)."""
         grid, block, smem = launch_shape(name, dims)
         fn = self.kernel(name)
-        descs, keep = _pack_params(args)
+        descs, keep = _pack_params(args, signature_types(name))
         n = rounds if mode == 0 else 1
         out = (C.c_float * n)()
         self.rt.imexHipProfileKernel(self.handle, fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
@@ -413,13 +467,19 @@ def flash_attention(stream, q, k, v, zh, n_ctx, sm_scale, queries_per_workgroup=
             stream.free(p)
 
 
-def mfma_lds_ceiling(stream, workgroups, iters, zero=False):
-    """The measurement kernel imex_mfma_lds_ceiling_f16 (no counterpart in the reference):
-    returns the one f32 per lane it stores, shape (workgroups, 512)."""
+def mfma_lds_ceiling(stream, workgroups, iters, mode=0):
+    """The measurement kernel imex_mfma_lds_ceiling_f16 (no counterpart in the reference; it lives in
+    lib/imex_probe.hsaco, outside the catalogue): returns the one f32 per lane it stores, shape
+    (workgroups, 512).  mode 0: operands uniform in (-1, 1) like the GEMM benchmark's; 1: zeros;
+    2: every f16 exponent below 1.0 equally likely."""
     n = workgroups * 512
-    d_o = stream.alloc(max(n, 1) * 4)
+    if workgroups < 1:
+        raise ValueError("at least one workgroup")
+    d_o = stream.alloc(n * 4)
     try:
-        stream.launch("imex_mfma_lds_ceiling_f16", [n], [d_o, n, int(iters), 1 if zero else 0])
+        fn = stream.kernel_from_file(PROBE_CODE_OBJECT, "imex_mfma_lds_ceiling_f16")
+        descs, keep = _pack_params([d_o, n, int(iters), int(mode)])
+        stream.rt.gpuLaunchKernel(stream.handle, fn, workgroups, 1, 1, 512, 1, 1, 0, C.cast(descs, C.c_void_p), None)
         stream.wait()
         return stream.from_device(d_o, (workgroups, 512), np.float32)
     finally:

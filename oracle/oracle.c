@@ -752,3 +752,19 @@ double oracle_time_gemm_rows(const void *A, const void *B, int64_t nrows, int64_
   free(rows);
   return 1e3 * (t1 - t0);
 }
+/* The MLP layer on the first nrows rows: the GEMM loop, then bias + SiLU + rounding to bf16. */
+double oracle_time_mlp_rows(const void *A, const void *B, const float *bias, int64_t nrows, int64_t N, int64_t K) {
+  int64_t *rows = (int64_t *)malloc((size_t)nrows * sizeof(int64_t));
+  for (int64_t i = 0; i < nrows; ++i) rows[i] = i;
+  float *C = (float *)calloc((size_t)(nrows * N), sizeof(float));
+  uint16_t *out = (uint16_t *)malloc((size_t)(nrows * N) * sizeof(uint16_t));
+  double t0 = now_s();
+  oracle_gemm_rows(A, B, C, rows, nrows, N, K, ORACLE_BF16);
+  oracle_bias_silu_bf16(C, bias, out, nrows, N);
+  double t1 = now_s();
+  g_sink = (float)out[0];
+  free(out);
+  free(C);
+  free(rows);
+  return 1e3 * (t1 - t0);
+}

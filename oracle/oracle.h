@@ -140,6 +140,7 @@ double oracle_time_softmax_f16(const uint16_t *x, int64_t rows, int64_t cols, in
 double oracle_time_rowsum_f32(const float *x, int64_t rows, int64_t cols, int warmup, int runs);
 double oracle_time_transpose2d(const void *x, int64_t rows, int64_t cols, int elem_bytes, int warmup, int runs);
 double oracle_time_gemm_rows(const void *A, const void *B, int64_t nrows, int64_t N, int64_t K, int ab_dtype);
+double oracle_time_mlp_rows(const void *A, const void *B, const float *bias, int64_t nrows, int64_t N, int64_t K);
 
 #ifdef __cplusplus
 }

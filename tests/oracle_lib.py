@@ -48,7 +48,7 @@ def lib():
             fn = getattr(_lib, "oracle_stat_" + name)
             fn.restype = C.c_float
             fn.argtypes = [C.c_void_p, C.c_size_t]
-        for name in ("relu_f32", "silu_f32", "softmax_f16", "rowsum_f32", "transpose2d", "gemm_rows"):
+        for name in ("relu_f32", "silu_f32", "softmax_f16", "rowsum_f32", "transpose2d", "gemm_rows", "mlp_rows"):
             getattr(_lib, "oracle_time_" + name).restype = C.c_double
     return _lib
 
@@ -397,3 +397,10 @@ def time_gemm_rows(a, b, nrows, ab_dtype):
     a, b = _c(a), _c(b)
     return lib().oracle_time_gemm_rows(_p(a), _p(b), C.c_int64(nrows), C.c_int64(b.shape[1]), C.c_int64(a.shape[1]),
                                        DT[ab_dtype])
+
+
+def time_mlp_rows(a, b, bias, nrows):
+    """ms for the first `nrows` rows of bf16(silu(A.B + bias)): the GEMM loop and the epilogue."""
+    a, b, bias = _c(a), _c(b), _c(bias, np.float32)
+    return lib().oracle_time_mlp_rows(_p(a), _p(b), _p(bias), C.c_int64(nrows), C.c_int64(b.shape[1]),
+                                      C.c_int64(a.shape[1]))

@@ -966,7 +966,7 @@ def test_gemm_f16_output_variant(host, orc, stream):
 
 
 # ==================== MFMA ceiling measurement kernel ======================
-def _ceiling_lds_f16(workgroup):
+def _ceiling_lds_f16(workgroup, mode):
     """The f16 operands imex_mfma_lds_ceiling_f16 writes into LDS, as (4096 slots, 8)."""
     with np.errstate(over="ignore"):
         i = np.arange(16384, dtype=np.uint32)
@@ -974,24 +974,29 @@ def _ceiling_lds_f16(workgroup):
         x ^= x >> np.uint32(15)
         x *= np.uint32(2246822519)
         x ^= x >> np.uint32(13)
-    lo = (x & np.uint32(0x83ff)) | (((x >> np.uint32(10)) % np.uint32(15)) << np.uint32(10))
-    hi = ((x >> np.uint32(16)) & np.uint32(0x83ff)) | (((x >> np.uint32(26)) % np.uint32(15)) << np.uint32(10))
+    if mode == 2:
+        lo = (x & np.uint32(0x83ff)) | (((x >> np.uint32(10)) % np.uint32(15)) << np.uint32(10))
+        hi = ((x >> np.uint32(16)) & np.uint32(0x83ff)) | (((x >> np.uint32(26)) % np.uint32(15)) << np.uint32(10))
+    else:
+        half = lambda h: (h.astype(np.float32) * np.float32(1.0 / 32768.0) - np.float32(1.0)).astype(np.float16).view(np.uint16).astype(np.uint32)
+        lo, hi = half(x & np.uint32(0xffff)), half(x >> np.uint32(16))
     words = lo | (hi << np.uint32(16))
     return words.view(np.uint16).view(np.float16).astype(np.float64).reshape(4096, 8)
 
 
-def test_mfma_ceiling_kernel_computes_what_it_says(host, stream):
+@pytest.mark.parametrize("mode", [0, 2])
+def test_mfma_ceiling_kernel_computes_what_it_says(host, stream, mode):
     """No oracle and no reference counterpart: the expected sums follow from the published
     operand / accumulator lane layout of MFMA 16x16x32 (A[m = l%16][k = 8(l/16)..+8],
     B likewise in n, C[4(l/16) + r][l%16] in register r), in f64."""
     iters, groups = 5, 3
     say("mfma ceiling probe: %d workgroups x %d steps" % (groups, iters))
-    got = host.mfma_lds_ceiling(stream, groups, iters)
+    got = host.mfma_lds_ceiling(stream, groups, iters, mode=mode)
     assert got.shape == (groups, 512)
     l = np.arange(64)
     rows = 4 * (l[:, None] // 16) + np.arange(4)[None, :]                      # [lane, r]
     for g in range(groups):
-        slots = _ceiling_lds_f16(g)
+        slots = _ceiling_lds_f16(g, mode)
         for w in range(8):
             lane = w * 64 + l
             total = np.zeros(64)
@@ -1012,5 +1017,5 @@ def test_mfma_ceiling_kernel_computes_what_it_says(host, stream):
             want = total
             have = got[g, w * 64:(w + 1) * 64].astype(np.float64)
             assert np.all(np.abs(have - want) <= 1e-4 * np.abs(want).max() + 1e-4), (g, w)
-    assert not np.any(host.mfma_lds_ceiling(stream, 2, 7, zero=True))
+    assert not np.any(host.mfma_lds_ceiling(stream, 2, 7, mode=1))
     assert host.mfma_lds_ceiling(stream, 1, 0).shape == (1, 512) and not np.any(host.mfma_lds_ceiling(stream, 1, 0))

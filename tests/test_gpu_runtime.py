@@ -177,6 +177,78 @@ def test_mgpu_entry_points(host, orc):
     rt.mgpuStreamDestroy(s)
 
 
+@pytest.mark.parametrize("bits", [32, 16])
+def test_memset_entry_points(host, bits):
+    """gpuMemSet32 / gpuMemSet16 (stream first) and mgpuMemset16: fills that start and end off the
+    16-byte grid, a length of zero, and what lies on either side of the filled range left alone."""
+    np_t = np.uint32 if bits == 32 else np.uint16
+    value = 0xdeadbeef if bits == 32 else 0xbf80  # bf16 -1.0
+    with host.Stream() as s:
+        for n, first in ((1, 0), (7, 3), (4096, 1), (100003, 5), ((1 << 21) + 9, 2)):
+            size = n + first + 11
+            back = np.arange(size, dtype=np.int64).astype(np_t)
+            d = s.to_device(back)
+            s.memset(int(d) + first * back.itemsize, value, n, bits=bits)
+            s.memset(int(d), 0x1234, 0, bits=bits)  # nothing to do
+            s.wait()
+            got = s.from_device(d, (size,), np_t)
+            assert np.all(got[first:first + n] == np_t(value)), (n, first)
+            assert np.array_equal(got[:first], back[:first]) and np.array_equal(got[first + n:], back[first + n:]), (n, first)
+            s.free(d)
+        if bits == 16:
+            d = s.alloc(2 * 1000)
+            host.runtime().mgpuMemset16(int(d), 0x3c00, 1000, s.handle)  # f16 1.0
+            s.wait()
+            assert np.all(s.from_device(d, (1000,), np.uint16) == 0x3c00)
+            s.free(d)
+
+
+def test_timestamp_handles_recycle(host, orc):
+    """Timestamps live in a 1024-slot ring per stream: recording thousands of them does not grow the
+    queue, and the two most recent ones still time the launches between them."""
+    n = 1 << 20
+    with host.Stream() as s:
+        d_in, d_out = s.to_device(orc.fill_uniform(n, "f32", 4, -1, 1)), s.alloc(n * 4)
+        step = s.prepare("imex_relu_f32", [n], [d_in, d_out, n])
+        seen = set()
+        for _ in range(3000):
+            seen.add(s.timestamp())
+        assert len(seen) == 1024
+        t0 = s.timestamp()
+        for _ in range(20):
+            step()
+        t1 = s.timestamp()
+        s.wait()
+        assert 0.0 < s.elapsed_ms(t0, t1) < 100.0
+        s.free(d_in)
+        s.free(d_out)
+
+
+def test_elapsed_time_refuses_launch_events():
+    """A launch event is an ordering point without a time of its own: imexHipEventElapsedMs takes
+    timestamps only, and says so through the ABI's error convention (message on stdout, abort)."""
+    prog = ("import sys; sys.path.insert(0, %r)\nimport __graft_entry__ as e\nimport numpy as np\n"
+            "host = e.load_package().host\ns = host.Stream()\nd = s.alloc(4096)\n"
+            "ev = s.launch('imex_relu_f32', [1024], [d, d, 1024])\nt = s.timestamp()\ns.wait()\n"
+            "print('before', flush=True)\ns.elapsed_ms(ev, t)\nprint('not reached')\n" % REPO)
+    r = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert r.returncode != 0
+    assert "before" in r.stdout and "not reached" not in r.stdout
+    assert "An exception was thrown: imexHipEventElapsedMs: both events must come from imexHipRecordTimestamp" in r.stdout
+
+
+def test_profiling_env_zero_warmups():
+    """IMEX_PROFILING_WARMUPS=0 means no warm-up launches (LevelZeroRuntimeWrappers.cpp:547-551), not the default."""
+    prog = ("import sys; sys.path.insert(0, %r)\nimport __graft_entry__ as e\nimport numpy as np\n"
+            "host = e.load_package().host\ns = host.Stream()\n"
+            "y = host.relu(s, np.linspace(-1, 1, 5000).astype(np.float32))\nprint('result', float(y.sum()))\n" % REPO)
+    env = dict(os.environ, IMEX_ENABLE_PROFILING="1", IMEX_PROFILING_RUNS="4", IMEX_PROFILING_WARMUPS="0")
+    r = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                       timeout=300, env=env)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert sum("execution time" in l and l.endswith("(over 4 runs)") for l in r.stdout.splitlines()) == 1
+
+
 def test_driver_report_mode(tmp_path):
     """The C++ driver in bench_imex's role: one child process per workload, their
     "execution time" lines collected in a report file (benchmarks/bench_imex.in:72-91)."""
