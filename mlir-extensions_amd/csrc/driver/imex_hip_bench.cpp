@@ -13,7 +13,7 @@
 // runtime):avg: ..." line per workload, the line bench_imex greps into
 // report.txt (bench_imex.in:87-91).
 //
-//   imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--launch-only N] <workload>...
+//   imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--rotate S] [--launch-only N] <workload>...
 //   imex-hip-bench --list
 //   imex-hip-bench [-l] --report report.txt <workload>...|all
 //
@@ -24,6 +24,9 @@
 //   -l             accepted for bench_imex compatibility (the HIP runtime is the only backend here)
 //   --zeros        all-zero inputs instead of random ones: MFMA power, and with it the clock the
 //                  part sustains, depends on operand values; this shows the kernel at full clock
+//   --rotate S     S separate copies of the workload's tensors, launches walking round them: with S x footprint
+//                  beyond the 256 MiB Infinity Cache every launch streams from HBM (back-to-back figure and
+//                  --launch-only runs; the per-launch statistics stay on the first set)
 //   --launch-only  skip the timing loop and just launch the kernel N times (for
 //                  rocprofv3 counter runs, which time and count every dispatch themselves)
 //
@@ -204,7 +207,7 @@ std::string programDir() {
 }
 
 struct Options {
-  int runs = 100, warmups = 10, launchOnly = 0;
+  int runs = 100, warmups = 10, launchOnly = 0, rotate = 1;
   bool flush = false, zeros = false;
 };
 
@@ -253,28 +256,49 @@ int runWorkload(const Workload &w, const Options &opt) {
   void *module = gpuModuleLoad(stream, blob, blobSize);
   void *kernel = gpuKernelGet(stream, module, w.kernel);
 
-  // ParamDesc list: pointers, then i64 scalars, then the optional f32 init; {NULL,0} ends it.
+  // Further copies of the tensors for --rotate: set s holds its own buffers, inputs copied from set 0.
+  std::vector<std::vector<void *>> sets(1, dev);
+  for (int s = 1; s < opt.rotate; ++s) {
+    std::vector<void *> more;
+    for (size_t t = 0; t < w.tensors.size(); ++t) {
+      const size_t bytes = static_cast<size_t>(count(w.tensors[t])) * elemBytes(w.tensors[t].elem);
+      more.push_back(gpuMemAlloc(stream, bytes, 64, /*isShared=*/0));
+      if (w.tensors[t].isInput)
+        gpuMemCopy(stream, more.back(), dev[t], bytes);
+    }
+    sets.push_back(more);
+  }
+
+  // ParamDesc list per set: pointers, then i64 scalars, then the optional f32 init; {NULL,0} ends it.
   std::vector<int64_t> idx(w.indexArgs);
   float init = 0.0f, scale = 0.5f;
-  std::vector<ImexParamDesc> params;
-  for (void *&p : dev)
-    params.push_back({&p, sizeof(void *)});
-  if (w.floatArg == 2)
-    params.push_back({&scale, sizeof(float)});
-  for (int64_t &v : idx)
-    params.push_back({&v, sizeof(int64_t)});
-  if (w.floatArg == 1)
-    params.push_back({&init, sizeof(float)});
-  params.push_back({nullptr, 0});
+  std::vector<std::vector<ImexParamDesc>> paramSets;
+  for (std::vector<void *> &set : sets) {
+    std::vector<ImexParamDesc> ps;
+    for (void *&p : set)
+      ps.push_back({&p, sizeof(void *)});
+    if (w.floatArg == 2)
+      ps.push_back({&scale, sizeof(float)});
+    for (int64_t &v : idx)
+      ps.push_back({&v, sizeof(int64_t)});
+    if (w.floatArg == 1)
+      ps.push_back({&init, sizeof(float)});
+    ps.push_back({nullptr, 0});
+    paramSets.push_back(ps);
+  }
+  std::vector<ImexParamDesc> &params = paramSets[0];
   ImexEventDesc noDeps[1] = {{nullptr}};
+  auto launch = [&](int i) {
+    gpuLaunchKernel(stream, kernel, grid[0], grid[1], grid[2], block[0], block[1], block[2], smem,
+                    paramSets[static_cast<size_t>(i) % paramSets.size()].data(), noDeps);
+  };
 
   if (opt.launchOnly > 0) {
     for (int i = 0; i < opt.launchOnly; ++i)
-      gpuLaunchKernel(stream, kernel, grid[0], grid[1], grid[2], block[0], block[1], block[2], smem, params.data(),
-                      noDeps);
+      launch(i);
     gpuWait(stream);
-    printf("%s: launched %s %d times, grid (%zu,%zu,%zu) block (%zu,%zu,%zu)\n", w.name, w.kernel, opt.launchOnly,
-           grid[0], grid[1], grid[2], block[0], block[1], block[2]);
+    printf("%s: launched %s %d times over %d buffer set(s), grid (%zu,%zu,%zu) block (%zu,%zu,%zu)\n", w.name, w.kernel,
+           opt.launchOnly, opt.rotate, grid[0], grid[1], grid[2], block[0], block[1], block[2]);
   } else {
     std::vector<float> times(opt.runs);
     imexHipProfileKernel(stream, kernel, grid[0], grid[1], grid[2], block[0], block[1], block[2], smem, params.data(),
@@ -282,21 +306,34 @@ int runWorkload(const Workload &w, const Options &opt) {
     float s[9];
     imexHipComputeStats(times.data(), times.size(), s);
     float total = 0.0f;
-    imexHipProfileKernel(stream, kernel, grid[0], grid[1], grid[2], block[0], block[1], block[2], smem, params.data(),
-                         opt.warmups, opt.runs, 0, 1, &total);
+    if (opt.rotate > 1) {
+      for (int i = 0; i < opt.warmups; ++i)
+        launch(i);
+      void *t0 = imexHipRecordTimestamp(stream);
+      for (int i = 0; i < opt.runs; ++i)
+        launch(opt.warmups + i);
+      void *t1 = imexHipRecordTimestamp(stream);
+      gpuWait(stream);
+      total = imexHipEventElapsedMs(t0, t1);
+    } else {
+      imexHipProfileKernel(stream, kernel, grid[0], grid[1], grid[2], block[0], block[1], block[2], smem, params.data(),
+                           opt.warmups, opt.runs, 0, 1, &total);
+    }
     const double backToBackMs = total / opt.runs;
     printf("%s: the kernel execution time is (ms, on HIP runtime):avg: %.4f, min: %.4f, max: %.4f, median: %4f, "
            "std_deviation: %4f, variance: %4f, P95: %4f, P5: %4f, median_one_third_avg: %4f (over %d runs)\n",
            w.name, s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], s[8], opt.runs);
     const double rate = w.work / (backToBackMs * (w.mfma ? 1e9 : 1e6));
-    printf("%s: back-to-back %.4f ms/launch = %.1f %s (%.1f%% of the %s roofline)%s\n", w.name, backToBackMs, rate,
+    printf("%s: back-to-back %.4f ms/launch = %.1f %s (%.1f%% of the %s roofline)%s%s\n", w.name, backToBackMs, rate,
            w.mfma ? "TFLOP/s" : "GB/s", 100.0 * rate / (w.mfma ? 2500.0 : 8000.0), w.mfma ? "2.5 PFLOP/s MFMA" : "8 TB/s HBM",
-           opt.flush ? " [per-launch times above measured after a cache flush]" : (opt.zeros ? " [all-zero inputs]" : ""));
+           opt.flush ? " [per-launch times above measured after a cache flush]" : (opt.zeros ? " [all-zero inputs]" : ""),
+           opt.rotate > 1 ? (" [rotating over " + std::to_string(opt.rotate) + " buffer sets]").c_str() : "");
   }
   fflush(stdout);
 
-  for (void *p : dev)
-    gpuMemFree(stream, p);
+  for (std::vector<void *> &set : sets)
+    for (void *p : set)
+      gpuMemFree(stream, p);
   gpuStreamDestroy(stream);
   return 0;
 }
@@ -371,6 +408,9 @@ int main(int argc, char **argv) {
       childOptions += " --warmups " + std::to_string(opt.warmups);
     } else if (a == "--launch-only" && i + 1 < argc) {
       opt.launchOnly = atoi(argv[++i]);
+    } else if (a == "--rotate" && i + 1 < argc) {
+      opt.rotate = atoi(argv[++i]);
+      childOptions += " --rotate " + std::to_string(opt.rotate);
     } else if (a == "all") {
       for (const Workload &w : all)
         names.push_back(w.name);
@@ -378,8 +418,8 @@ int main(int argc, char **argv) {
       names.push_back(a);
     }
   }
-  if (names.empty() || opt.runs < 1) {
-    fprintf(stderr, "usage: imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--launch-only N] [--report FILE] <workload>|all ...\n"
+  if (names.empty() || opt.runs < 1 || opt.rotate < 1 || opt.rotate > 64) {
+    fprintf(stderr, "usage: imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--rotate S] [--launch-only N] [--report FILE] <workload>|all ...\n"
                     "       imex-hip-bench --list\n");
     return 2;
   }

@@ -15,8 +15,9 @@
 //    faster on tensors that sit in the caches, the same when they stream from HBM.
 //  * rows of up to 4096 elements: a workgroup owns a row and stages it in LDS
 //    as f32 (read once, three passes over LDS).
-//  * longer rows, or bases that break 16-byte alignment on the register path:
-//    workgroup per row, re-reading the row from cache.
+//  * longer rows: workgroup per row, the streaming form -- a running (max, sum)
+//    pair rescaled as the maximum moves, then a second read of the row to
+//    normalise (WG/softmax_intra_sg_cross_lane.mlir:135-175): two reads, one write.
 // Internals are f32; 16-bit I/O follows the reference's policy for 16-bit types
 // on the GPU: extend to f32, compute, truncate (docs/Transforms/BF16ToGpu.md:17-26).
 //
@@ -260,22 +261,78 @@ __device__ __forceinline__ void softmax_row_in_lds(const void *in, void *out, in
   __syncthreads(); // rowBuf is reused by the next row
 }
 
-// ---- any length: workgroup per row, three passes over the (cached) input ----------------
+// ---- any length: workgroup per row, the input read twice -----------------------------------
+// The streaming form of test/Integration/Dialect/XeGPU/WG/softmax_intra_sg_cross_lane.mlir:135-175:
+// one pass carries a running maximum m and a running sum s of exp(x - m), rescaling s by
+// exp(m_old - m_new) whenever the maximum moves; a second pass over the input normalises.  Here a
+// lane moves its maximum once per 16-byte vector (one rescale per vector, not per element), and the
+// lanes' (m, s) pairs are merged the same way: S = sum_i s_i exp(m_i - M), M = max_i m_i.
+struct RunningSoftmax {
+  float m = kMaxInit, s = 0.0f;
+  template <int N> __device__ __forceinline__ void add(const float (&x)[N]) {
+    float mx = m;
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      mx = fmaxf(mx, x[i]);
+    float t = s * fast_exp(m - mx); // m == mx: exp(0) = 1; first vector: s = 0
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      t += fast_exp(x[i] - mx); // a NaN element, which fmaxf passes over, makes the sum NaN here
+    m = mx;
+    s = t;
+  }
+};
+
 template <Dt D>
 __device__ __forceinline__ void softmax_row_streamed(const void *in, void *out, int64_t row, int64_t cols,
-                                                     float *scratch) {
+                                                     float *scratch, bool vec) {
   using E = Elem<D>;
   const int64_t base = row * cols;
-  float m = kMaxInit;
-  for (int64_t c = threadIdx.x; c < cols; c += kThreads)
-    m = fmaxf(m, E::load(in, base + c));
-  m = block_reduce(m, true, scratch);
-  float s = 0.0f;
-  for (int64_t c = threadIdx.x; c < cols; c += kThreads)
-    s += fast_exp(E::load(in, base + c) - m);
-  s = block_reduce(s, false, scratch);
-  for (int64_t c = threadIdx.x; c < cols; c += kThreads)
-    E::store(out, base + c, fast_exp(E::load(in, base + c) - m) / s);
+  const int64_t vecs = cols / E::kPerVec;
+  const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(in) + base * E::kBytes);
+  RunningSoftmax run;
+  if (vec) {
+    // two vectors in flight per lane
+    int64_t v = threadIdx.x;
+    for (; v + kThreads < vecs; v += 2 * kThreads) {
+      const u32x4 r0 = src[v], r1 = src[v + kThreads];
+      float f0[E::kPerVec], f1[E::kPerVec];
+      E::unpack(r0, f0);
+      E::unpack(r1, f1);
+      run.add(f0);
+      run.add(f1);
+    }
+    if (v < vecs) {
+      float f[E::kPerVec];
+      E::unpack(src[v], f);
+      run.add(f);
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < cols; c += kThreads) {
+      const float f[1] = {E::load(in, base + c)};
+      run.add(f);
+    }
+  }
+  // merge the 256 running pairs: the row maximum, then every lane's sum brought to it
+  const float m = block_reduce(run.m, true, scratch);
+  const float sum = block_reduce(run.s * fast_exp(run.m - m), false, scratch);
+  // one IEEE division per row, then multiplies (an f32 rounding away from z / s at most); a sum of
+  // zero (a row of -inf) gives 0 * inf = NaN like the 0 / 0 of the reference's division
+  const float inv = 1.0f / sum;
+  if (vec) {
+    u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + base * E::kBytes);
+    for (int64_t v = threadIdx.x; v < vecs; v += kThreads) {
+      float f[E::kPerVec];
+      E::unpack(src[v], f);
+#pragma unroll
+      for (int i = 0; i < E::kPerVec; ++i)
+        f[i] = fast_exp(f[i] - m) * inv;
+      dst[v] = E::pack(f);
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < cols; c += kThreads)
+      E::store(out, base + c, fast_exp(E::load(in, base + c) - m) * inv);
+  }
 }
 
 template <Dt D>
@@ -296,7 +353,7 @@ __device__ __forceinline__ void softmax_kernel(const void *in, void *out, int64_
       softmax_row_in_lds<D>(in, out, row, cols, rowBuf, scratch, aligned);
   } else {
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x)
-      softmax_row_streamed<D>(in, out, row, cols, scratch);
+      softmax_row_streamed<D>(in, out, row, cols, scratch, aligned);
   }
 }
 

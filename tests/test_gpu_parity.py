@@ -186,6 +186,28 @@ def test_softmax_bf16_and_exact_rows(host, orc, stream):
     assert np.all(got[:, 5] == 1.0) and got.sum() == 4.0
 
 
+@pytest.mark.parametrize("rows,cols", [(3, 5000), (2, 65536 + 8), (5, 4097), (2, 300001)])
+def test_softmax_long_rows_streaming_form(host, orc, stream, rows, cols):
+    """Rows beyond 4096 columns take the running (max, sum) form of WG/softmax_intra_sg_cross_lane.mlir:135-175;
+    checked against the reference's scalar three-pass loop (:85-117) and the benchmark form, on random
+    rows, on a ramp whose maximum moves with every vector (every partial sum is rescaled again and
+    again), on its mirror image, and on one huge element at the very end."""
+    say("softmax streaming %dx%d" % (rows, cols))
+    x = orc.fill_normal(rows * cols, "f32", 81 + cols % 7, 0.0, 2.0).reshape(rows, cols).copy()
+    x[0] = np.linspace(-40.0, 30.0, cols, dtype=np.float32)  # outputs stay normal f32 numbers (the hardware exp flushes subnormal results)
+    x[1] = x[0][::-1]
+    if rows > 2:
+        x[2, -1] = 60.0
+    got = host.softmax(stream, x, "f32")
+    for ref in (orc.softmax_f32(x, three_pass=True), orc.softmax_f32(x)):
+        assert np.all(np.abs(got - ref) <= 1e-3 * np.abs(ref))  # the stated bar
+    # the sequential f32 sum of the reference loop carries up to ~2e-4 of rounding over 300 001 addends (it
+    # differs by that much between a row and its mirror image); against the exact row sum the kernel is tighter
+    assert np.max(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0)) < 2e-5
+    xh = orc.from_float(x, "f16")
+    assert close_16(orc, host.softmax(stream, xh, "f16"), orc.softmax_16(xh, "f16"), "f16")
+
+
 @pytest.mark.parametrize("dtype,cols", [("f32", 20), ("f32", 512), ("f16", 1024), ("f32", 3000), ("f16", 4096),
                                         ("f32", 5000), ("f16", 70000)])
 def test_softmax_nan_and_infinite_rows(host, orc, stream, dtype, cols):
