@@ -66,7 +66,8 @@ struct Workload {
   int floatArg;                 // 0 none; 1 trailing f32 `init` (reductions); 2 f32 between pointers and indices (sm_scale)
   double work;                  // algorithmic bytes or flops per launch
   bool mfma;                    // roofline: MFMA (TFLOP/s) or HBM (GB/s)
-  bool probe = false;           // a measurement kernel: loaded from imex_probe.hsaco beside this program, one lane per dims[0]
+  bool probe = false;           // a measurement kernel: loaded from imex_probe.hsaco beside this program
+  int probeGrid = 0;            // its grid (workgroups of 512 lanes); 0: one lane per dims[0]
 };
 
 std::vector<Workload> workloads() {
@@ -168,6 +169,19 @@ std::vector<Workload> workloads() {
        {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 0}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
       {"mfma_lds_ceiling_f16_zeros", "imex_mfma_lds_ceiling_f16", {256 * 512},
        {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 1}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
+      // the GEMM's tile code with one part switched off (timing only: the results are meaningless)
+      {"gemm_f16_4096_probe_no_loop_copies", "imex_gemm_probe_no_loop_copies", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_f16_4096_probe_no_epilogue", "imex_gemm_probe_no_epilogue", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_f16_4096_probe_multiply_only", "imex_gemm_probe_multiply_only", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_f16_4096_probe_copies_only", "imex_gemm_probe_copies_only", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
       {"mfma_lds_ceiling_f16_every_exponent", "imex_mfma_lds_ceiling_f16", {256 * 512},
        {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 2}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
   };
@@ -231,7 +245,7 @@ int runWorkload(const Workload &w, const Options &opt) {
   const void *blob = nullptr;
   static std::vector<char> probeBlob; // kept for the life of the process: the runtime caches modules by address
   if (w.probe) {
-    grid[0] = static_cast<size_t>((w.dims[0] + 511) / 512);
+    grid[0] = w.probeGrid ? static_cast<size_t>(w.probeGrid) : static_cast<size_t>((w.dims[0] + 511) / 512);
     if (probeBlob.empty()) {
       const std::string path = programDir() + "/imex_probe.hsaco";
       FILE *f = fopen(path.c_str(), "rb");

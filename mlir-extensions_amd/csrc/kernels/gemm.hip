@@ -1,540 +1,15 @@
-// Tiled MFMA GEMM for gfx950: C[M,N] = A[M,K] . B[K,N], A and B f16 or bf16
-// (row-major), f32 accumulate; also with A stored [K,M] or B stored [N,K].
-//
-// Reference kernels (workgroup-level XeGPU, the role XeTile's
-// load_tile / prefetch_tile / tile_mma played):
-//   test/Integration/Dialect/XeGPU/WG/gemm_4kx4kx4k_f16_f16_f32.mlir:47-91
-//     256x256 workgroup tile, K-step 32, three-deep prefetch, C += A.B;
-//   test/Integration/Dialect/XeGPU/WG/gemm_4kx4kx4k_f16_f16_f32_bias.mlir:77-116
-//     bias[n] broadcast over rows and added after the K loop;
-//   benchmarks/silu/silu_gpu.mlir.in:3-19 for the activation fused below;
-//   test/Integration/Dialect/XeGPU/WG/gemm_4kx4kx4k_transpose_{a,b}.mlir for the
-//     operand storage orders (the same kernel with the other operand loader).
-//
-// Blocking on MI355X:
-//   workgroup tile 256 x 256, 512 threads = 8 wavefronts in a 2 x 4 grid (two per
-//   SIMD), each owning 128 x 64 = 8 x 4 MFMA 16x16x32 blocks (128 accumulator
-//   registers).  16x16x32 rather than 32x32x16: the two read the same LDS bytes per
-//   FLOP, but on random operands the part sustains about 9 % more with the former
-//   (the shader clock under MFMA load follows the operand values);
-//   K advances 32 at a time through a ring of four 32 KiB LDS stages: A and B
-//   tiles go from global memory STRAIGHT into LDS (buffer_load ... lds, 16 bytes
-//   per lane, no register staging) three steps ahead of the step that multiplies
-//   them; a step waits (vmcnt) only for the oldest tile in flight, then meets the
-//   other wavefronts at the step's single barrier;
-//   the LDS images are swizzled -- A [256 rows][32 k] by 16-byte group, B
-//   [32 k][256 n] by 32-byte pair -- and because a direct copy fixes each lane's
-//   LDS position, the swizzle is applied to the lane's GLOBAL address instead;
-//   A fragments are 128-bit LDS reads; B is row-major [K,N] while the MFMA wants
-//   eight consecutive k per lane, so B fragments use the LDS transpose read
-//   (ds_read_b64_tr_b16) -- no permutes, no transposed copy of B anywhere;
-//   a K-step is multiplied in two halves of 16 MFMAs (the wavefront's upper, then
-//   lower four row blocks, each by all four column blocks); fragments are
-//   double-buffered in registers: the LDS reads the next half needs are placed by
-//   hand between the MFMAs of this one (sched_barrier fences keep the order), and
-//   the step's barrier sits between the halves so that sixteen MFMAs are always
-//   queued behind it;
-//   f32 results: the accumulator blocks of two neighbouring column blocks swap
-//   16-lane rows (v_permlane16_swap) so that every store instruction writes whole
-//   128-byte lines; 16-bit results: the product is taken transposed, which leaves
-//   four consecutive columns in a lane's registers -- one 8-byte store;
-//   workgroup ids are remapped so that the 32 workgroups resident on one XCD
-//   (ids congruent mod 8) cover a compact 4 x 8 block of tiles and share A and
-//   B panels in that XCD's L2.
-//
-// M and N need not divide the tile: edge tiles copy the last row / column that exists
-// in place of the missing ones and store only what is inside C.  What the MFMA path
-// does need is K in whole steps of 32 and 16-byte aligned rows in memory (N % 8 == 0
-// where B is [K,N], M % 8 == 0 where A is [K,M]); other shapes take the
-// one-thread-per-output path of the same kernels, which adds in ascending k like the
-// reference's CPU loop (lib/ExecutionEngine/ImexRunnerUtils.cpp:308-317).
+// Entry points of the tiled MFMA GEMM for gfx950: C[M,N] = A[M,K] . B[K,N], A and B f16 or bf16
+// (row-major), f32 accumulate; also with A stored [K,M] or B stored [N,K].  The tile code, its
+// blocking and the reference kernels it stands for are described in gemm_tile.h.
 //
 // Launch: block (512,1,1); grid (tiles,1,1) with tiles = ceil(M/256)*ceil(N/256) on
-// the MFMA path, else (ceil(M*N/512),1,1); workgroups stride, so any grid is correct.  The fixed-shape 4096^3 entry
-// points take the reference's own launch: blocks (16,16,1), threads (512,1,1).
+// the MFMA path, else (ceil(M*N/512),1,1); workgroups stride, so any grid is correct.  The fixed-shape
+// 4096^3 entry points take the reference's own launch: blocks (16,16,1), threads (512,1,1).
 
-#include "device_common.h"
+#include "gemm_tile.h"
 
 using namespace imexhip;
-
-namespace {
-
-// Wavefront grid inside the 256 x 256 workgroup tile: 2 x 4, each wavefront 128 x 64.
-constexpr int kWavesM = 2, kWavesN = 4;
-constexpr int kWaves = kWavesM * kWavesN;
-constexpr int kThreads = 64 * kWaves;
-constexpr int BM = 256, BN = 256;
-constexpr int RK = 32;                              // K per step (one ring stage)
-constexpr int WM = BM / kWavesM, WN = BN / kWavesN; // wavefront tile
-constexpr int FI = WM / 16, FJ = WN / 16;           // MFMA 16x16 tiles per wavefront: 8 x 4
-constexpr int kStages = 4;                          // LDS ring: 4 x 32 KiB of the 160 KiB
-constexpr int kImageBytes = 256 * RK * 2;           // one operand's 256 x 32 slab: 16 KiB
-constexpr int kRStage = 2 * kImageBytes;            // A image + B image
-constexpr int kDmaPerWave = kImageBytes / 1024 / kWaves; // 1 KiB global->LDS copies per wavefront, operand and step
-constexpr int kDist = kStages - 1;                  // tiles in flight ahead of the one being multiplied
-constexpr int kGroupM = 4;                          // tile rows per L2-sharing group
-
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));   // 4 floats at any float address
-typedef uint16_t u16x4u __attribute__((ext_vector_type(4), aligned(2))); // 4 halves at any half address
-typedef short i16x4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) i16x4 LdsI16x4; // operand type of the LDS transpose read
-typedef __attribute__((address_space(3))) char LdsChar;
-
-struct F16 {
-  using Frag = f16x8;
-  static __device__ __forceinline__ f32x4 mfma(Frag a, Frag b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ float widen(uint16_t h) { return half_bits_to_float(h); }
-};
-struct BF16 {
-  using Frag = bf16x8;
-  static __device__ __forceinline__ f32x4 mfma(Frag a, Frag b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ float widen(uint16_t h) { return bf16_bits_to_float(h); }
-};
-
-// Keeps the compiler's scheduler from moving anything across this point.
-#define IMEX_FENCE() __builtin_amdgcn_sched_barrier(0)
-
-// ---- epilogues ------------------------------------------------------------------
-// operator() takes one element of the accumulator.  kColumnsInRegisters picks how the tiled
-// path holds the accumulator: true = four consecutive columns of one row in a lane's four
-// registers, handed to vec4() (16-bit outputs: one 8-byte store per lane); false = one column
-// per lane, rows in the registers, stored element by element after the lane-row swap that
-// lines 32 consecutive columns up across lanes (32-bit outputs: whole 128-byte lines).
-struct StoreF32 {       // C = acc
-  static constexpr bool kColumnsInRegisters = false;
-  float *C;
-  __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
-    C[m * N + n] = acc; // ordinary store: C stays in the last-level cache for whoever reads it next
-  }
-};
-struct AccumulateF32 {  // C = C + acc   (the reference kernel loads C as its initial accumulator)
-  static constexpr bool kColumnsInRegisters = false;
-  float *C;
-  __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
-    C[m * N + n] = C[m * N + n] + acc;
-  }
-};
-struct BiasAccumulateF32 { // C = bias[n] + (C + acc)  (bias.mlir:88-94,112-113)
-  static constexpr bool kColumnsInRegisters = false;
-  float *C;
-  const float *bias;
-  __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
-    C[m * N + n] = bias[n] + (C[m * N + n] + acc);
-  }
-};
-// v / (1 + exp(-v)) with the hardware's exponential and reciprocal estimates (about an ulp each):
-// the result is rounded to bf16, 2^-9 relative, straight afterwards.
-__device__ __forceinline__ float silu_fast(float v) { return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
-
-// f32 -> bf16 by the hardware's conversion (round to nearest even; pairs become one v_cvt_pk_bf16_f32).
-// Numbers convert as float_to_bf16_bits does; a NaN keeps its leading payload bits instead of becoming
-// the canonical one.
-__device__ __forceinline__ uint16_t bf16_bits_hw(float f) { return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f)); }
-
-struct BiasSiluBF16 {   // out = bf16( silu( acc + bias[n] ) )
-  static constexpr bool kColumnsInRegisters = true;
-  uint16_t *out;
-  const float *bias;
-  __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
-    const float v = acc + bias[n];
-    const float y = silu_fast(v);
-    out[m * N + n] = bf16_bits_hw(y);
-  }
-  __device__ __forceinline__ void vec4(int64_t m, int64_t n, int64_t N, f32x4 acc) const {
-    const f32x4 b = *reinterpret_cast<const f32x4u *>(bias + n);
-    u16x4u o;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float v = acc[r] + b[r];
-      const float y = silu_fast(v);
-      o[r] = bf16_bits_hw(y);
-    }
-    *reinterpret_cast<u16x4u *>(out + m * N + n) = o;
-  }
-};
-struct StoreF16 {       // C(f16) = acc   (WG/gemm_4kx4kx4k_f16_f16_f16.mlir)
-  static constexpr bool kColumnsInRegisters = true;
-  uint16_t *C;
-  __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
-    C[m * N + n] = static_cast<uint16_t>(float_to_half_bits(acc));
-  }
-  __device__ __forceinline__ void vec4(int64_t m, int64_t n, int64_t N, f32x4 acc) const {
-    u16x4u o;
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      o[r] = static_cast<uint16_t>(float_to_half_bits(acc[r]));
-    *reinterpret_cast<u16x4u *>(C + m * N + n) = o;
-  }
-};
-
-// ---- one-thread-per-output path ---------------------------------------------------
-// kAT: A is stored [K,M] (A[k*M+m]) instead of [M,K]; kBT: B is stored [N,K]
-// (B[n*K+k]) instead of [K,N].
-template <typename T, bool kAT, bool kBT, typename Epi>
-__device__ __forceinline__ void gemm_scalar(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
-                                            Epi epi) {
-  // grid-stride, so that any launch shape covers every output
-  const int64_t block = int64_t(blockIdx.y) * gridDim.x + blockIdx.x;
-  const int64_t stride = int64_t(gridDim.x) * gridDim.y * kThreads;
-  for (int64_t idx = block * kThreads + threadIdx.x; idx < M * N; idx += stride) {
-    const int64_t m = idx / N, n = idx % N;
-    float acc = 0.0f;
-    for (int64_t k = 0; k < K; ++k) {
-      const float a = T::widen(kAT ? A[k * M + m] : A[m * K + k]);
-      const float b = T::widen(kBT ? B[n * K + k] : B[k * N + n]);
-      const float p = a * b;
-      acc = acc + p; // rounded multiply, rounded add (file is built with contraction off)
-    }
-    epi(m, n, N, acc);
-  }
-}
-
-// ---- tiled MFMA path ----------------------------------------------------------------
-// Buffer resource for raw buffer loads: base pointer, byte range, and the gfx9
-// "32-bit data format" word; out-of-range lanes read zeros.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, int64_t bytes) {
-  const int range = bytes > 0x7fffffff ? 0x7fffffff : int(bytes);
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, range, 0x00020000);
-}
-
-template <int N> __device__ __forceinline__ void wait_vmcnt() {
-  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
-}
-
-// One MFMA operand of a workgroup tile: a 256 x 32 (rows x k) slab per step.  Both
-// A (rows = m) and B (rows = n) want, per lane, row = lane % 16 of a 16-row
-// fragment and the 8 consecutive k starting at (lane / 16) * 8.
-//
-// KContig: the slab is k-contiguous in memory (A as [M,K], B as [N,K]).  LDS image
-//   [256 rows][32 k], 64-byte rows; 16-byte group c of row r is stored at group
-//   c ^ h((r >> 2) & 3), h = {0, 2, 3, 1}.  A fragment is one ds_read_b128 (lane: row
-//   lane % 16, group lane / 16); the LDS serves such a read 16 lanes at a time, and the
-//   lanes that go together are not neighbours (0-3 with 12-15, 20-23 and 24-27; 4-7 with
-//   8-11, 16-19 and 28-31; likewise in the upper half) -- h is chosen so that each of
-//   those sets touches every bank once.  One 1 KiB copy = 16 rows.
-// KStrided: the slab's rows are strided in memory (B as [K,N], A as [K,M]).  LDS
-//   image [32 k][256 rows], 512-byte rows; 32-byte pair p of k-row r at pair
-//   p ^ g(r), g(r) = (r & 3) | ((r >> 3 & 1) << 2).  One copy = 2 k-rows.  A
-//   fragment is two LDS transpose reads (ds_read_b64_tr_b16): within each group of
-//   16 lanes, lane t supplies the address of 4 consecutive rows at k-row t/4 and
-//   receives 4 consecutive k of row t.
-// A direct global->LDS copy puts lane l's 16 bytes at base + 16 l, so the swizzle
-// is applied to the lane's GLOBAL address instead.
-__device__ __forceinline__ int kcontig_swizzle(int row) { return (0x78 >> (((row >> 2) & 3) * 2)) & 3; }
-
-template <typename T, bool kStrided, int kFrags> struct Operand {
-  __amdgpu_buffer_rsrc_t rsrc;
-  int voff[kDmaPerWave];         // per-lane byte offset of each copy at step 0
-  int step;                      // bytes per K-step in memory
-  int dstWave;                   // LDS byte offset of this wavefront's copies inside the image
-  int rd[kStrided ? kFrags : 1]; // per-lane LDS read bases: KStrided one per fragment, KContig one (fragments 1 KiB apart)
-
-  // ptr: the operand's matrix; ld: its leading dimension; first: first row (m0 or n0)
-  // of the slab; w0: the wavefront's first row inside the slab; extent: rows * cols.
-  // A slab that sticks out of the matrix (last tile row / column of a ragged shape): the
-  // lanes that would copy rows past the end copy the last row that exists instead, so no
-  // address ever leaves the matrix; those rows only feed outputs that are never stored.
-  __device__ __forceinline__ void setup(const uint16_t *ptr, int64_t ld, int64_t first, int w0, int64_t extent,
-                                        int wave, int lane) {
-    if constexpr (!kStrided) {
-      const int64_t rows = extent / ld - first; // rows of the matrix from `first` on, >= 1
-      const int last = rows < 256 ? int(rows) - 1 : 255;
-      rsrc = make_rsrc(ptr + first * ld, int64_t(last + 1) * ld * 2);
-#pragma unroll
-      for (int q = 0; q < kDmaPerWave; ++q) {
-        const int row = wave * (256 / kWaves) + q * 16 + (lane >> 2);
-        const int chunk = (lane & 3) ^ kcontig_swizzle(row);
-        voff[q] = int((int64_t(min(row, last)) * ld + chunk * 8) * 2);
-      }
-      step = RK * 2;
-      dstWave = wave * (256 / kWaves) * (RK * 2);
-      const int fragRow = lane & 15, kGroup = lane >> 4;
-      rd[0] = (w0 + fragRow) * (RK * 2) + ((kGroup ^ kcontig_swizzle(fragRow)) << 4);
-    } else {
-      rsrc = make_rsrc(ptr + first, (extent - first) * 2);
-#pragma unroll
-      for (int q = 0; q < kDmaPerWave; ++q) {
-        const int row = wave * (RK / kWaves) + q * 2 + (lane >> 5);
-        const int g = (row & 3) | (((row >> 3) & 1) << 2);
-        const int chunk = (((((lane & 31) >> 1) ^ g)) << 1) | (lane & 1);
-        const int64_t col = min(int64_t(chunk * 8), ld - 8 - first); // ld % 8 == 0: the last 16 bytes of the k-row
-        voff[q] = int((int64_t(row) * ld + col) * 2);
-      }
-      step = int(RK * ld * 2);
-      dstWave = wave * (RK / kWaves) * 512;
-      const int t = lane & 15, kGroup = lane >> 4;
-      const int g = (t >> 2) | ((kGroup & 1) << 2); // g(k-row) for k-row = kGroup*8 + h*4 + t/4
-      const int pair0 = w0 / 16;                    // 32-byte pair holding fragment 0's rows
-#pragma unroll
-      for (int f = 0; f < kFrags; ++f)
-        rd[f] = (kGroup * 8 + (t >> 2)) * 512 + (((pair0 + f) ^ g) * 32) + (t & 3) * 8;
-    }
-  }
-  // the wavefront's copies of K-step kt into the image at LDS byte offset `image`
-  __device__ __forceinline__ void dma(LdsChar *lds, int image, int kt) const {
-#pragma unroll
-    for (int q = 0; q < kDmaPerWave; ++q)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + image + dstWave + q * 1024, 16, voff[q], kt * step, 0, 0);
-  }
-  // fragment f (rows w0 + 16 f ..., all 32 k) of the image at `image`
-  __device__ __forceinline__ typename T::Frag read(const char *lds, int image, int f) const {
-    if constexpr (!kStrided) {
-      return *reinterpret_cast<const typename T::Frag *>(lds + image + rd[0] + f * 16 * (RK * 2));
-    } else {
-      const char *p = lds + image + rd[f];
-      const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p));           // k +0..3
-      const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4 *)(p + 4 * 512)); // k +4..7
-      return __builtin_bit_cast(typename T::Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-    }
-  }
-};
-
-// kAT / kBT as in gemm_scalar.  A is KContig unless transposed; B is KContig only
-// when transposed.
-// One 256 x 256 tile of C: tile number `id` of a tilesM x tilesN grid.
-template <typename T, bool kAT, bool kBT, typename Epi>
-__device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, int64_t M,
-                                          int64_t N, int64_t K, Epi epi, char *lds, int tilesM, int tilesN, int id) {
-  static_assert(FI == 8 && FJ == 4 && kWaves == 8, "written for 8 wavefronts of 8 x 4 MFMA tiles");
-  LdsChar *lds_base = (LdsChar *)lds;
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave / kWavesN, wn = wave % kWavesN;
-
-  // -- tile number -> tile, XCD-aware -------------------------------------------------
-  const int tiles = tilesM * tilesN;
-  int pid = id;
-  if (tiles % 8 == 0)
-    pid = (pid % 8) * (tiles / 8) + pid / 8; // ids congruent mod 8 share an XCD
-  const int group = kGroupM * tilesN;
-  const int firstM = (pid / group) * kGroupM;
-  const int groupRows = min(tilesM - firstM, kGroupM);
-  const int tileM = firstM + (pid % group) % groupRows;
-  const int tileN = (pid % group) / groupRows;
-  const int64_t m0 = int64_t(tileM) * BM, n0 = int64_t(tileN) * BN;
-
-  const int waveU = __builtin_amdgcn_readfirstlane(wave);
-  Operand<T, kAT, FI> opA;
-  Operand<T, !kBT, FJ> opB;
-  opA.setup(A, kAT ? M : K, m0, wm * WM, M * K, waveU, lane);
-  opB.setup(B, kBT ? K : N, n0, wn * WN, K * N, waveU, lane);
-  constexpr int kImgA = 0, kImgB = kImageBytes;
-  auto dma_tile = [&](int kt, int stageOff) { // stageOff: byte offset of the ring stage, wave-uniform
-    opA.dma(lds_base, stageOff + kImgA, kt);
-    opB.dma(lds_base, stageOff + kImgB, kt);
-  };
-
-  // acc[i][j] is the 16 x 16 block at rows 16 i, columns 16 j of the wavefront's tile, held
-  // TRANSPOSED (the MFMA is given the B fragment as its first operand): lane l has row
-  // l % 16 and the four consecutive columns (l / 16) * 4 ..., which is one 16-byte store.
-  f32x4 acc[FI][FJ];
-#pragma unroll
-  for (int i = 0; i < FI; ++i)
-#pragma unroll
-    for (int j = 0; j < FJ; ++j)
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        acc[i][j][r] = 0.0f;
-
-  // A step multiplies the wavefront's upper four row fragments (half 0), then the lower four
-  // (half 1), each by all four B fragments.  af[h] holds half h's A fragments; bf[p] the B
-  // fragments of a step of parity p.
-  typename T::Frag af[2][FI / 2], bf[2][FJ];
-  auto read_a = [&](int stageOff, int h, int ii) { af[h][ii] = opA.read(lds, stageOff + kImgA, h * (FI / 2) + ii); };
-  auto read_b = [&](int stageOff, int p, int j) { bf[p][j] = opB.read(lds, stageOff + kImgB, j); };
-  auto mm = [&](int h, int p, int ii, int j) {
-    if constexpr (Epi::kColumnsInRegisters)
-      acc[h * (FI / 2) + ii][j] = T::mfma(bf[p][j], af[h][ii], acc[h * (FI / 2) + ii][j]);
-    else
-      acc[h * (FI / 2) + ii][j] = T::mfma(af[h][ii], bf[p][j], acc[h * (FI / 2) + ii][j]);
-  };
-  // half 0 of a step of parity p: 16 MFMAs, and between them the reads of this step's lower
-  // A fragments (the fences keep the compiler from regrouping them).  The MFMAs go column
-  // block by column block, up and down the row blocks in turn, so that one operand at most
-  // changes from one MFMA to the next (fewer operand bits switching: about 1 % on random data).
-  auto half0 = [&](int p, int curOff) {
-#pragma unroll
-    for (int j = 0; j < FJ; ++j) {
-#pragma unroll
-      for (int s = 0; s < FI / 2; ++s) {
-        mm(0, p, (j & 1) ? FI / 2 - 1 - s : s, j);
-        if (s == 0) read_a(curOff, 1, j);
-        IMEX_FENCE();
-      }
-    }
-  };
-  // half 1: 16 MFMAs, and between them the reads of the NEXT step's upper A fragments and
-  // of its B fragments (into the other parity's registers)
-  auto half1 = [&](int p, int nxtOff) {
-#pragma unroll
-    for (int j = 0; j < FJ; ++j) {
-#pragma unroll
-      for (int s = 0; s < FI / 2; ++s) {
-        mm(1, p, (j & 1) ? FI / 2 - 1 - s : s, j);
-        if (s == 0) read_a(nxtOff, 0, j);
-        if (s == 2) read_b(nxtOff, p ^ 1, j);
-        IMEX_FENCE();
-      }
-    }
-  };
-
-  const int kTiles = int(K / RK);
-  const int lastTile = kTiles - 1;
-  // prologue: tiles 0 .. kDist-1 in flight, tile 0 landed, its first fragments in registers
-#pragma unroll
-  for (int t = 0; t < kDist; ++t)
-    dma_tile(min(t, lastTile), t * kRStage);
-  wait_vmcnt<(kDist - 1) * 2 * kDmaPerWave>();
-  __builtin_amdgcn_s_barrier();
-  IMEX_FENCE();
-#pragma unroll
-  for (int ii = 0; ii < FI / 2; ++ii) read_a(0, 0, ii);
-#pragma unroll
-  for (int j = 0; j < FJ; ++j) read_b(0, 0, j);
-  IMEX_FENCE();
-
-  int curOff = 0;               // stage of tile t
-  int nxtOff = kRStage;         // stage of tile t+1
-  int dmaOff = kDist * kRStage; // stage tile t+kDist goes to (= stage of tile t-1)
-  auto step = [&](int p, int t) {
-    // The stage of tile t-1 is free: every wavefront passed the previous step's
-    // barrier after its last reads of it.  Past the end of K the copies re-fetch the
-    // last tile into a stage nobody reads, so every step is the same code.
-    dma_tile(min(t + kDist, lastTile), dmaOff);
-    IMEX_FENCE();
-    half0(p, curOff);                               // rows 0-63 of tile t; reads its rows 64-127
-    wait_vmcnt<(kDist - 1) * 2 * kDmaPerWave>();    // tile t+1 has landed (this wavefront's part) ...
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();                   // ... and everyone else's; all reads of tile t are done
-    IMEX_FENCE();
-    half1(p, nxtOff);                               // rows 64-127 of tile t; reads tile t+1's rows 0-63 and B
-    curOff = nxtOff;
-    nxtOff = nxtOff + kRStage == kStages * kRStage ? 0 : nxtOff + kRStage;
-    dmaOff = dmaOff + kRStage == kStages * kRStage ? 0 : dmaOff + kRStage;
-  };
-  int t = 0;
-  for (; t + 1 < kTiles; t += 2) { // two steps per trip, so that the B registers' parity is a literal
-    step(0, t);
-    step(1, t + 1);
-  }
-  if (t < kTiles)
-    step(0, t);
-  wait_vmcnt<0>();
-
-  // -- epilogue.  kColumnsInRegisters: lane holds, for block (i,j), row lane%16 and columns
-  //    (lane/16)*4 + 0..3; otherwise column lane%16 and rows (lane/16)*4 + 0..3.
-  const bool interior = m0 + BM <= M && n0 + BN <= N; // uniform over the workgroup: nothing to mask
-  if constexpr (Epi::kColumnsInRegisters) {
-    const int64_t mBase = m0 + wm * WM + (lane & 15), nBase = n0 + wn * WN + (lane >> 4) * 4;
-    if (interior) {
-#pragma unroll
-      for (int i = 0; i < FI; ++i)
-#pragma unroll
-        for (int j = 0; j < FJ; ++j)
-          epi.vec4(mBase + i * 16, nBase + j * 16, N, acc[i][j]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < FI; ++i)
-#pragma unroll
-        for (int j = 0; j < FJ; ++j)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int64_t m = mBase + i * 16, n = nBase + j * 16 + r;
-            if (m < M && n < N)
-              epi(m, n, N, acc[i][j][r]);
-          }
-    }
-  } else {
-    // Blocks j and j+1 sit side by side in C.  Swapping the odd 16-lane rows of one with the
-    // even rows of the other leaves lanes 0-31 of a register with 32 consecutive columns of
-    // one row of C and lanes 32-63 with the row 8 below: whole 128-byte lines per store.
-    const int64_t mBase = m0 + wm * WM + (lane >> 5) * 8, nBase = n0 + wn * WN + (lane & 31);
-    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); // the last MFMA results are in their registers
-#pragma unroll
-    for (int i = 0; i < FI; ++i)
-#pragma unroll
-      for (int j = 0; j < FJ; j += 2)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          // (written as an instruction: the compiler's own handling of the corresponding builtin
-          // lost track of the second result here; the waits on either side stand in for the
-          // hazard padding the compiler would add)
-          asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1"
-                       : "+v"(acc[i][j][r]), "+v"(acc[i][j + 1][r])); // -> rows r, r+8 | rows r+4, r+12
-        }
-    if (interior) {
-#pragma unroll
-      for (int i = 0; i < FI; ++i)
-#pragma unroll
-        for (int j = 0; j < FJ; j += 2)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            epi(mBase + i * 16 + r, nBase + j * 16, N, acc[i][j][r]);
-            epi(mBase + i * 16 + r + 4, nBase + j * 16, N, acc[i][j + 1][r]);
-          }
-    } else {
-#pragma unroll
-      for (int i = 0; i < FI; ++i)
-#pragma unroll
-        for (int j = 0; j < FJ; j += 2)
-#pragma unroll
-          for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int64_t m = mBase + i * 16 + r + 4 * h, n = nBase + j * 16;
-              if (m < M && n < N)
-                epi(m, n, N, acc[i][j + h][r]);
-            }
-    }
-  }
-}
-
-// Workgroups stride over the tiles: a launch with fewer workgroups than tiles still covers C, one
-// with more leaves the surplus nothing to do.
-template <typename T, bool kAT, bool kBT, typename Epi>
-__device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
-                                           int64_t M, int64_t N, int64_t K, Epi epi, char *lds) {
-  const int tilesM = int((M + BM - 1) / BM), tilesN = int((N + BN - 1) / BN);
-  const int tiles = tilesM * tilesN, workgroups = gridDim.x * gridDim.y;
-  for (int id = blockIdx.y * gridDim.x + blockIdx.x; id < tiles; id += workgroups) {
-    gemm_tile<T, kAT, kBT, Epi>(A, B, M, N, K, epi, lds, tilesM, tilesN, id);
-    if (id + workgroups < tiles)
-      __syncthreads(); // the ring is reused by this workgroup's next tile
-  }
-}
-
-template <typename T, bool kAT, bool kBT, typename Epi>
-__device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
-                                           Epi epi) {
-  // 4 stages x (256 + 256) rows x 32 k x 2 B = 128 KiB of the CU's 160 KiB LDS.
-  __shared__ __attribute__((aligned(16))) char lds[kStages * kRStage];
-  // The MFMA path wants K in whole 32-wide steps and 16-byte aligned rows in memory: a row of
-  // B [K,N] (or of A [K,M] when transposed) is N (M) elements long, so those must be multiples
-  // of 8.  M and N need not divide the tile: edge tiles multiply padding and store what exists.
-  // An operand whose rows are strided in memory is addressed with 32-bit byte offsets from one
-  // buffer descriptor, so it has to stay below 2 GiB; a k-contiguous one below 4 Mi elements per row.
-  constexpr int64_t kMaxBytes = int64_t(1) << 31, kMaxRow = int64_t(1) << 22;
-  const bool fitsA = kAT ? K * M * 2 < kMaxBytes : K < kMaxRow;
-  const bool fitsB = kBT ? K < kMaxRow : K * N * 2 < kMaxBytes;
-  const bool tileable = M > 0 && N > 0 && K > 0 && K % RK == 0 && (kBT || N % 8 == 0) && (!kAT || M % 8 == 0) &&
-                        fitsA && fitsB &&
-                        ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
-  if (tileable)
-    gemm_tiled<T, kAT, kBT, Epi>(A, B, M, N, K, epi, lds);
-  else
-    gemm_scalar<T, kAT, kBT, Epi>(A, B, M, N, K, epi);
-}
-
-} // namespace
+using namespace imexhip_gemm;
 
 // C = A.B
 extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_f16_f16_f32(const uint16_t *A, const uint16_t *B,

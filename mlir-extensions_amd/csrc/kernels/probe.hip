@@ -1,6 +1,12 @@
-//===- probe.hip - what the MFMA pipe sustains on given operand values ------===//
+//===- probe.hip - measurement kernels (bench-only code object) --------------===//
 //
-// A measurement kernel, not an operator (no counterpart in the reference): the
+// Not operators and not in the catalogue (no counterpart in the reference):
+//  * imex_mfma_lds_ceiling_f16: what the MFMA pipe sustains on given operand values;
+//  * imex_gemm_probe_*: the tiled GEMM's own tile code (gemm_tile.h) with one part switched
+//    off -- the K loop's global -> LDS copies, the epilogue, both, or everything but the
+//    copies -- to price each part on the benchmark's operands.  Their results are meaningless.
+//
+// imex_mfma_lds_ceiling_f16: the
 // inner product loop of the tiled GEMM with everything but the matrix pipe and
 // its LDS operand reads taken away -- no global loads, no barriers in the loop,
 // no epilogue beyond one store per lane.
@@ -36,6 +42,7 @@
 //===----------------------------------------------------------------------===//
 
 #include "device_common.h"
+#include "gemm_tile.h"
 
 namespace {
 
@@ -100,3 +107,14 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_mfma_lds_ceiling_f16
   if (idx < outCount)
     out[idx] = s;
 }
+
+// ---- the GEMM's tile code with parts switched off (arguments and launch as imex_gemm_f16_f16_f32) ----
+#define IMEX_GEMM_PROBE(name, switches)                                                                               \
+  extern "C" __global__ __launch_bounds__(imexhip_gemm::kThreads) void name(                                          \
+      const uint16_t *A, const uint16_t *B, float *C, int64_t M, int64_t N, int64_t K) {                              \
+    imexhip_gemm::gemm_entry<imexhip_gemm::F16, false, false, (switches)>(A, B, M, N, K, imexhip_gemm::StoreF32{C});  \
+  }
+IMEX_GEMM_PROBE(imex_gemm_probe_no_loop_copies, imexhip_gemm::kProbeNoLoopCopies)
+IMEX_GEMM_PROBE(imex_gemm_probe_no_epilogue, imexhip_gemm::kProbeNoEpilogue)
+IMEX_GEMM_PROBE(imex_gemm_probe_multiply_only, imexhip_gemm::kProbeNoLoopCopies | imexhip_gemm::kProbeNoEpilogue)
+IMEX_GEMM_PROBE(imex_gemm_probe_copies_only, imexhip_gemm::kProbeCopiesOnly)

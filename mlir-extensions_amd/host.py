@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
+import re
 
 import numpy as np
 
@@ -167,7 +168,7 @@ def signature_types(kernel):
     k = kernels()
     for i in range(k.imexHipKernelCount()):
         if k.imexHipKernelName(i).decode() == kernel:
-            sig = k.imexHipKernelSignature(i).decode().strip()[1:-1]
+            sig = re.sub(r"\[[^\]]*\]", "", k.imexHipKernelSignature(i).decode().strip()[1:-1])  # drop layout notes "[K,M]"
             types = []
             for part in sig.split(","):
                 t = part.split(":", 1)[1].strip()
