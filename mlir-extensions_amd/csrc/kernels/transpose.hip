@@ -8,14 +8,14 @@
 //
 // Here a workgroup moves a tile through LDS so that both the HBM reads and the
 // HBM writes are 128-bit per lane and contiguous per row segment:
-//  * 32-bit: R x C tile in tile[R][C+1] words; the odd pitch makes the row-wise
-//    scalar LDS writes and the column-wise scalar LDS reads conflict-free.
-//  * 16-bit: R x 128 tile (or two of them side by side, loaded together).  Two
-//    vertically adjacent rows are interleaved in
-//    registers into 32-bit words (in[2p][c], in[2p+1][c]) -- two neighbouring
-//    elements of output row c -- and stored transposed; output rows then leave
-//    LDS as 128-bit reads.  The 16-byte groups of each LDS row are XOR-swizzled
-//    with the column group so neither side has bank conflicts.
+//  * 32-bit: R x C tile kept transposed in LDS in 16-byte groups of four input
+//    rows; a lane's four row loads give it a 4 x 4 block that it transposes by
+//    picking components, so both LDS sides are 128-bit accesses, XOR-swizzled by
+//    group so neither side has bank conflicts.
+//  * 16-bit: R x 128 tile (or two of them side by side, loaded together), the
+//    same scheme on 8 x 8 blocks: a lane's eight row loads are repacked with
+//    v_perm_b32 into eight 128-bit groups of the transposed image, one per
+//    column; 128-bit LDS accesses on both sides, XOR-swizzled by group.
 //  * Tile size: the WRITE side of a transpose is the scattered one, and its row
 //    segments are R elements long.  Measured streaming from HBM, 512-byte write
 //    segments reach 74-78% of peak where 256-byte ones stop at 67-70%, so large
@@ -52,93 +52,109 @@ struct View {
 };
 
 // ---- 32-bit elements: R x C tile ----------------------------------------------------
+// LDS holds the tile TRANSPOSED, T[C][R] words, in 16-byte groups of four consecutive input rows.
+// A lane loads four consecutive rows (4 b .. 4 b + 3) at four consecutive columns (4 v .. 4 v + 3),
+// one 128-bit load per row with whole 512-byte row segments per wavefront; the 4 x 4 block is then
+// transposed by picking components -- no data moves between lanes -- and goes to LDS as four 128-bit
+// writes, T[4 v + k][group b].  Output rows leave LDS as 128-bit reads of consecutive groups.  Group g
+// of row c is kept at position g ^ ((c / 4) % 16): the sixteen lanes an LDS access serves together then
+// touch sixteen different 16-byte bank groups on the write side (consecutive v) and on the read side
+// (consecutive g) alike.
 template <int R, int C>
 __device__ __forceinline__ void tile32_fast(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
-                                            const View &v, int64_t r0, int64_t c0, uint32_t (*tile)[C + 1]) {
-  constexpr int VR = C / 4, RP = kThreads / VR, LP = R / RP; // load: vectors per row, rows per pass, passes
-  const int cv = threadIdx.x % VR, rr = threadIdx.x / VR;
-  u32x4 x[LP];
+                                            const View &v, int64_t r0, int64_t c0, u32x4 *tile) {
+  constexpr int VR = C / 4, BP = kThreads / VR, LP = R / 4 / BP; // load: vectors per row, row blocks per pass, passes
+  constexpr int G = R / 4;                                      // 16-byte groups per LDS row
+  static_assert(G >= 16 && (G & (G - 1)) == 0 && LP >= 1, "the group swizzle needs at least 16 groups per row");
+  const int cv = threadIdx.x % VR, bb = threadIdx.x / VR;
+  u32x4 x[LP][4];
 #pragma unroll
   for (int p = 0; p < LP; ++p) {
-    const int r = rr + RP * p;
-    if (r0 + r < v.rows && c0 + cv * 4 < v.cols)
-      x[p] = load128<true>(reinterpret_cast<const u32x4 *>(in + (r0 + r) * v.ldIn + c0 + cv * 4));
+    const int b = bb + BP * p; // row block: input rows 4 b .. 4 b + 3
+    if (r0 + 4 * b < v.rows && c0 + cv * 4 < v.cols) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        x[p][j] = load128<true>(reinterpret_cast<const u32x4 *>(in + (r0 + 4 * b + j) * v.ldIn + c0 + cv * 4));
+    }
   }
 #pragma unroll
   for (int p = 0; p < LP; ++p) {
-    const int r = rr + RP * p;
-    tile[r][cv * 4 + 0] = x[p].x;
-    tile[r][cv * 4 + 1] = x[p].y;
-    tile[r][cv * 4 + 2] = x[p].z;
-    tile[r][cv * 4 + 3] = x[p].w;
+    const int b = bb + BP * p;
+    const int pos = b ^ (cv & 15); // (c / 4) % 16 is the same for the four columns of this vector
+    tile[(cv * 4 + 0) * G + pos] = u32x4{x[p][0].x, x[p][1].x, x[p][2].x, x[p][3].x};
+    tile[(cv * 4 + 1) * G + pos] = u32x4{x[p][0].y, x[p][1].y, x[p][2].y, x[p][3].y};
+    tile[(cv * 4 + 2) * G + pos] = u32x4{x[p][0].z, x[p][1].z, x[p][2].z, x[p][3].z};
+    tile[(cv * 4 + 3) * G + pos] = u32x4{x[p][0].w, x[p][1].w, x[p][2].w, x[p][3].w};
   }
   __syncthreads();
-  constexpr int VO = R / 4, CP = kThreads / VO, SP = C / CP; // store: vectors per output row, rows per pass, passes
-  const int iv = threadIdx.x % VO, cc = threadIdx.x / VO;    // 4 input rows -> one output vector
+  constexpr int CP = kThreads / G, SP = C / CP; // store: output rows per pass, passes
+  const int g = threadIdx.x % G, cc = threadIdx.x / G;
 #pragma unroll
   for (int p = 0; p < SP; ++p) {
     const int c = cc + CP * p; // output row within the tile
-    if (c0 + c < v.cols && r0 + iv * 4 < v.rows) {
-      u32x4 y = {tile[iv * 4 + 0][c], tile[iv * 4 + 1][c], tile[iv * 4 + 2][c], tile[iv * 4 + 3][c]};
-      store128<true>(y, reinterpret_cast<u32x4 *>(out + (c0 + c) * v.ldOut + r0 + iv * 4));
-    }
+    if (c0 + c < v.cols && r0 + g * 4 < v.rows)
+      store128<true>(tile[c * G + (g ^ ((c >> 2) & 15))], reinterpret_cast<u32x4 *>(out + (c0 + c) * v.ldOut + r0 + g * 4));
   }
 }
 
-// ---- 16-bit elements: R x 128 tile ------------------------------------------------------
-// LDS image: [128 output rows][R/2 words]; word w of output row c holds input
-// rows 2w, 2w+1 at column c.  16-byte group g of row c is stored at group
-// g ^ (c/8).
-template <int R> __device__ __forceinline__ int swz16(int col, int rowPair) {
-  constexpr int W = R / 2; // words per output row
-  return col * W + ((((rowPair >> 2) ^ (col >> 3)) & (W / 4 - 1)) << 2) + (rowPair & 3);
-}
-
-// kHalves = 2: the tile is R x 256; the loads of both 128-column halves are issued
-// together (512-byte row segments on the read side as well), then each half takes
-// its turn through the LDS image.
+// ---- 16-bit elements: R x 128 tile (or two of them side by side) ---------------------------
+// The same scheme as the 32-bit tile with blocks of 8 x 8 elements: a lane loads eight consecutive rows
+// (8 b .. 8 b + 7) at eight consecutive columns, one 128-bit load per row; for each of its eight columns it
+// packs the eight row values into four words (v_perm_b32 on the words of two adjacent rows) and writes
+// them as one 128-bit group of the transposed LDS image T[128 columns][R elements].  Output rows leave
+// LDS as 128-bit reads.  Group g of LDS row c sits at position g ^ ((c / 8) % 16).
+// kHalves = 2: the tile is R x 256; the loads of both 128-column halves are issued together (512-byte row
+// segments on the read side as well), then each half takes its turn through the LDS image.
 template <int R, int kHalves>
 __device__ __forceinline__ void tile16_fast(const uint16_t *__restrict__ in, uint16_t *__restrict__ out,
-                                            const View &v, int64_t r0, int64_t c0, uint32_t *words) {
-  constexpr int LP = R / 32; // 16 row pairs per pass
-  const int cg = threadIdx.x % 16; // 8-element column group
-  const int rq = threadIdx.x / 16; // row pair within a pass
-  u32x4 a[kHalves][LP], b[kHalves][LP];
+                                            const View &v, int64_t r0, int64_t c0, u32x4 *tile) {
+  constexpr int G = R / 8;               // 16-byte groups per LDS row
+  constexpr int BP = kThreads / 16;      // row blocks per pass (16 column groups of 8 across 128 columns)
+  constexpr int LP = G / BP;             // passes
+  static_assert(G >= 16 && (G & (G - 1)) == 0 && LP >= 1, "the group swizzle needs at least 16 groups per row");
+  const int cg = threadIdx.x % 16, bb = threadIdx.x / 16;
+  u32x4 x[kHalves][LP][8];
 #pragma unroll
-  for (int pass = 0; pass < LP; ++pass) {
-    const int rp = rq + 16 * pass;
+  for (int p = 0; p < LP; ++p) {
+    const int b = bb + BP * p; // input rows 8 b .. 8 b + 7
 #pragma unroll
     for (int h = 0; h < kHalves; ++h)
-      if (r0 + 2 * rp < v.rows && c0 + h * 128 + cg * 8 < v.cols) {
-        const uint16_t *p = in + (r0 + 2 * rp) * v.ldIn + c0 + h * 128 + cg * 8;
-        a[h][pass] = load128<true>(reinterpret_cast<const u32x4 *>(p));
-        b[h][pass] = load128<true>(reinterpret_cast<const u32x4 *>(p + v.ldIn));
+      if (r0 + 8 * b < v.rows && c0 + h * 128 + cg * 8 < v.cols) {
+        const uint16_t *src = in + (r0 + 8 * b) * v.ldIn + c0 + h * 128 + cg * 8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          x[h][p][j] = load128<true>(reinterpret_cast<const u32x4 *>(src + j * v.ldIn));
       }
   }
-  constexpr int VO = R / 8, CP = kThreads / VO, SP = 128 / CP; // vectors per output row, rows per pass, passes
-  const int g = threadIdx.x % VO; // 8 consecutive input rows
+  constexpr int CP = kThreads / G, SP = 128 / CP; // store: output rows per pass, passes
+  const int g = threadIdx.x % G, cc = threadIdx.x / G;
 #pragma unroll
   for (int h = 0; h < kHalves; ++h) {
     if (h > 0)
       __syncthreads(); // the previous half has left LDS
 #pragma unroll
-    for (int pass = 0; pass < LP; ++pass) {
-      const int rp = rq + 16 * pass;
+    for (int p = 0; p < LP; ++p) {
+      const int pos = (bb + BP * p) ^ cg; // (c / 8) % 16 = cg for this lane's eight columns
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        // even column: low halves of both rows; odd column: high halves
-        words[swz16<R>(cg * 8 + 2 * k, rp)] = __builtin_amdgcn_perm(b[h][pass][k], a[h][pass][k], 0x05040100u);
-        words[swz16<R>(cg * 8 + 2 * k + 1, rp)] = __builtin_amdgcn_perm(b[h][pass][k], a[h][pass][k], 0x07060302u);
+      for (int m = 0; m < 4; ++m) {
+        // column 2 m of the group: the low halves of word m of each row; column 2 m + 1: the high halves
+        u32x4 lo, hi;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          lo[q] = __builtin_amdgcn_perm(x[h][p][2 * q + 1][m], x[h][p][2 * q][m], 0x05040100u);
+          hi[q] = __builtin_amdgcn_perm(x[h][p][2 * q + 1][m], x[h][p][2 * q][m], 0x07060302u);
+        }
+        tile[(cg * 8 + 2 * m) * G + pos] = lo;
+        tile[(cg * 8 + 2 * m + 1) * G + pos] = hi;
       }
     }
     __syncthreads();
 #pragma unroll
-    for (int pass = 0; pass < SP; ++pass) {
-      const int c = threadIdx.x / VO + CP * pass; // output row within this half
-      if (c0 + h * 128 + c < v.cols && r0 + g * 8 < v.rows) {
-        u32x4 y = *reinterpret_cast<const u32x4 *>(words + swz16<R>(c, g * 4));
-        store128<true>(y, reinterpret_cast<u32x4 *>(out + (c0 + h * 128 + c) * v.ldOut + r0 + g * 8));
-      }
+    for (int p = 0; p < SP; ++p) {
+      const int c = cc + CP * p; // output row within this half
+      if (c0 + h * 128 + c < v.cols && r0 + g * 8 < v.rows)
+        store128<true>(tile[c * G + (g ^ ((c >> 3) & 15))],
+                       reinterpret_cast<u32x4 *>(out + (c0 + h * 128 + c) * v.ldOut + r0 + g * 8));
     }
   }
 }
@@ -187,8 +203,8 @@ template <typename T>
 __device__ __forceinline__ void transpose_block(const T *in, T *out, const View &v, int64_t planes, int64_t inPlane,
                                                 int64_t outPlane) {
   constexpr int kVec = 16 / sizeof(T);
-  // 32-bit: 128 x 129 words = 66048 B.  16-bit: 128 rows x 128 words = 65536 B.
-  constexpr int kLdsBytes = sizeof(T) == 4 ? 128 * 129 * 4 : 128 * 128 * 4;
+  // 32-bit: 128 x 128 words.  16-bit: 128 rows x 128 words.  The scalar path's 64 x 65 elements fit as well.
+  constexpr int kLdsBytes = 128 * 128 * 4;
   __shared__ __attribute__((aligned(16))) char lds[kLdsBytes];
   const bool fast = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
                     v.rows % kVec == 0 && v.cols % kVec == 0 && v.ldIn % kVec == 0 && v.ldOut % kVec == 0 &&
@@ -201,22 +217,20 @@ __device__ __forceinline__ void transpose_block(const T *in, T *out, const View 
   } else if constexpr (sizeof(T) == 4) {
     if (big)
       for_each_tile<128, 128>(v, planes, [&](int64_t plane, int64_t r0, int64_t c0) {
-        tile32_fast<128, 128>(in + plane * inPlane, out + plane * outPlane, v, r0, c0,
-                              reinterpret_cast<uint32_t(*)[129]>(lds));
+        tile32_fast<128, 128>(in + plane * inPlane, out + plane * outPlane, v, r0, c0, reinterpret_cast<u32x4 *>(lds));
       });
     else
       for_each_tile<64, 64>(v, planes, [&](int64_t plane, int64_t r0, int64_t c0) {
-        tile32_fast<64, 64>(in + plane * inPlane, out + plane * outPlane, v, r0, c0,
-                            reinterpret_cast<uint32_t(*)[65]>(lds));
+        tile32_fast<64, 64>(in + plane * inPlane, out + plane * outPlane, v, r0, c0, reinterpret_cast<u32x4 *>(lds));
       });
   } else {
     if (big)
       for_each_tile<256, 256>(v, planes, [&](int64_t plane, int64_t r0, int64_t c0) {
-        tile16_fast<256, 2>(in + plane * inPlane, out + plane * outPlane, v, r0, c0, reinterpret_cast<uint32_t *>(lds));
+        tile16_fast<256, 2>(in + plane * inPlane, out + plane * outPlane, v, r0, c0, reinterpret_cast<u32x4 *>(lds));
       });
     else
       for_each_tile<128, 128>(v, planes, [&](int64_t plane, int64_t r0, int64_t c0) {
-        tile16_fast<128, 1>(in + plane * inPlane, out + plane * outPlane, v, r0, c0, reinterpret_cast<uint32_t *>(lds));
+        tile16_fast<128, 1>(in + plane * inPlane, out + plane * outPlane, v, r0, c0, reinterpret_cast<u32x4 *>(lds));
       });
   }
 }
