@@ -15,7 +15,7 @@
 //
 //   imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--rotate S] [--launch-only N] <workload>...
 //   imex-hip-bench --list
-//   imex-hip-bench [-l] --report report.txt <workload>...|all
+//   imex-hip-bench [-l] --report report.txt <workload>...|all|operators
 //
 //   --report FILE  bench_imex's outer loop (bench_imex.in:72-91): one child process per workload,
 //                  their output echoed, every "execution time" line collected in FILE under an
@@ -425,9 +425,10 @@ int main(int argc, char **argv) {
     } else if (a == "--rotate" && i + 1 < argc) {
       opt.rotate = atoi(argv[++i]);
       childOptions += " --rotate " + std::to_string(opt.rotate);
-    } else if (a == "all") {
+    } else if (a == "all" || a == "operators") { // operators: everything but the measurement kernels
       for (const Workload &w : all)
-        names.push_back(w.name);
+        if (a == "all" || !w.probe)
+          names.push_back(w.name);
     } else {
       names.push_back(a);
     }
