@@ -45,8 +45,9 @@
 //
 // M and N need not divide the tile: edge tiles copy the last row / column that exists
 // in place of the missing ones and store only what is inside C.  What the MFMA path
-// does need is K in whole steps of 32 and 16-byte aligned rows in memory (N % 8 == 0
-// where B is [K,N], M % 8 == 0 where A is [K,M]); other shapes take the
+// does need is 16-byte aligned rows in memory (K % 8 == 0; N % 8 == 0
+// where B is [K,N], M % 8 == 0 where A is [K,M]; a K that does not fill the last 32-wide step is
+// padded with zeros on the way into LDS); other shapes take the
 // one-thread-per-output path of the same kernels, which adds in ascending k like the
 // reference's CPU loop (lib/ExecutionEngine/ImexRunnerUtils.cpp:308-317).
 //
@@ -241,9 +242,16 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 // is applied to the lane's GLOBAL address instead.
 __device__ __forceinline__ int kcontig_swizzle(int row) { return (0x78 >> (((row >> 2) & 3) * 2)) & 3; }
 
-template <typename T, bool kStrided, int kFrags> struct Operand {
+// kTail: K is not a multiple of the 32-wide step; the copies of the last step then use a second set of
+// offsets in which every 16-byte piece that lies at k >= K is sent out of the buffer's range -- such a
+// lane fetches nothing and its 16 bytes of LDS are written with zeros, so the step multiplies zeros
+// there.  (An offset beyond the range, not a skipped lane: the LDS image must not keep stale values.)
+constexpr int kOutOfRange = 0x7ffffff0;
+
+template <typename T, bool kStrided, int kFrags, bool kTail> struct Operand {
   __amdgpu_buffer_rsrc_t rsrc;
   int voff[kDmaPerWave];         // per-lane byte offset of each copy at step 0
+  int voffTail[kTail ? kDmaPerWave : 1]; // the same for the last, partial step
   int step;                      // bytes per K-step in memory
   int dstWave;                   // LDS byte offset of this wavefront's copies inside the image
   int rd[kStrided ? kFrags : 1]; // per-lane LDS read bases: KStrided one per fragment, KContig one (fragments 1 KiB apart)
@@ -253,8 +261,9 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
   // A slab that sticks out of the matrix (last tile row / column of a ragged shape): the
   // lanes that would copy rows past the end copy the last row that exists instead, so no
   // address ever leaves the matrix; those rows only feed outputs that are never stored.
+  // kRem: the k the last step still holds (8 .. 32; 32 unless kTail)
   __device__ __forceinline__ void setup(const uint16_t *ptr, int64_t ld, int64_t first, int w0, int64_t extent,
-                                        int wave, int lane) {
+                                        int wave, int lane, int kRem) {
     if constexpr (!kStrided) {
       const int64_t rows = extent / ld - first; // rows of the matrix from `first` on, >= 1
       const int last = rows < 256 ? int(rows) - 1 : 255;
@@ -264,6 +273,8 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
         const int row = wave * (256 / kWaves) + q * 16 + (lane >> 2);
         const int chunk = (lane & 3) ^ kcontig_swizzle(row);
         voff[q] = int((int64_t(min(row, last)) * ld + chunk * 8) * 2);
+        if constexpr (kTail)
+          voffTail[q] = chunk * 8 < kRem ? voff[q] : kOutOfRange;
       }
       step = RK * 2;
       dstWave = wave * (256 / kWaves) * (RK * 2);
@@ -278,6 +289,8 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
         const int chunk = (((((lane & 31) >> 1) ^ g)) << 1) | (lane & 1);
         const int64_t col = min(int64_t(chunk * 8), ld - 8 - first); // ld % 8 == 0: the last 16 bytes of the k-row
         voff[q] = int((int64_t(row) * ld + col) * 2);
+        if constexpr (kTail)
+          voffTail[q] = row < kRem ? voff[q] : kOutOfRange;
       }
       step = int(RK * ld * 2);
       dstWave = wave * (RK / kWaves) * 512;
@@ -289,11 +302,16 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
         rd[f] = (kGroup * 8 + (t >> 2)) * 512 + (((pair0 + f) ^ g) * 32) + (t & 3) * 8;
     }
   }
-  // the wavefront's copies of K-step kt into the image at LDS byte offset `image`
-  __device__ __forceinline__ void dma(LdsChar *lds, int image, int kt) const {
+  // the wavefront's copies of K-step kt into the image at LDS byte offset `image`; partial: kt is the
+  // last step of a K that does not fill it (uniform over the wavefront)
+  __device__ __forceinline__ void dma(LdsChar *lds, int image, int kt, bool partial) const {
 #pragma unroll
-    for (int q = 0; q < kDmaPerWave; ++q)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + image + dstWave + q * 1024, 16, voff[q], kt * step, 0, 0);
+    for (int q = 0; q < kDmaPerWave; ++q) {
+      int v = voff[q];
+      if constexpr (kTail)
+        v = partial ? voffTail[q] : v;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + image + dstWave + q * 1024, 16, v, kt * step, 0, 0);
+    }
   }
   // fragment f (rows w0 + 16 f ..., all 32 k) of the image at `image`
   __device__ __forceinline__ typename T::Frag read(const char *lds, int image, int f) const {
@@ -311,7 +329,7 @@ template <typename T, bool kStrided, int kFrags> struct Operand {
 // kAT / kBT as in gemm_scalar.  A is KContig unless transposed; B is KContig only
 // when transposed.
 // One 256 x 256 tile of C: tile number `id` of a tilesM x tilesN grid.
-template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0>
+template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0, bool kTail = false>
 __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, int64_t M,
                                           int64_t N, int64_t K, Epi epi, char *lds, int tilesM, int tilesN, int id) {
   static_assert(FI == 8 && FJ == 4 && kWaves == 8, "written for 8 wavefronts of 8 x 4 MFMA tiles");
@@ -334,14 +352,18 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   const int64_t m0 = int64_t(tileM) * BM, n0 = int64_t(tileN) * BN;
 
   const int waveU = __builtin_amdgcn_readfirstlane(wave);
-  Operand<T, kAT, FI> opA;
-  Operand<T, !kBT, FJ> opB;
-  opA.setup(A, kAT ? M : K, m0, wm * WM, M * K, waveU, lane);
-  opB.setup(B, kBT ? K : N, n0, wn * WN, K * N, waveU, lane);
+  const int kTiles = int((K + RK - 1) / RK);
+  const int lastTile = kTiles - 1;
+  const int kRem = int(K - int64_t(lastTile) * RK); // k in the last step: 32, or 8 / 16 / 24 with kTail
+  Operand<T, kAT, FI, kTail> opA;
+  Operand<T, !kBT, FJ, kTail> opB;
+  opA.setup(A, kAT ? M : K, m0, wm * WM, M * K, waveU, lane, kRem);
+  opB.setup(B, kBT ? K : N, n0, wn * WN, K * N, waveU, lane, kRem);
   constexpr int kImgA = 0, kImgB = kImageBytes;
   auto dma_tile = [&](int kt, int stageOff) { // stageOff: byte offset of the ring stage, wave-uniform
-    opA.dma(lds_base, stageOff + kImgA, kt);
-    opB.dma(lds_base, stageOff + kImgB, kt);
+    const bool partial = kTail && kt == lastTile;
+    opA.dma(lds_base, stageOff + kImgA, kt, partial);
+    opB.dma(lds_base, stageOff + kImgB, kt, partial);
   };
 
   // acc[i][j] is the 16 x 16 block at rows 16 i, columns 16 j of the wavefront's tile, held
@@ -410,8 +432,6 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
     }
   };
 
-  const int kTiles = int(K / RK);
-  const int lastTile = kTiles - 1;
   // prologue: tiles 0 .. kDist-1 in flight, tile 0 landed, its first fragments in registers
   if constexpr (kProbe & kProbeNoLoopCopies) { // every stage filled once, with real operand values
 #pragma unroll
@@ -541,13 +561,13 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
 
 // Workgroups stride over the tiles: a launch with fewer workgroups than tiles still covers C, one
 // with more leaves the surplus nothing to do.
-template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0>
+template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0, bool kTail = false>
 __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                            int64_t M, int64_t N, int64_t K, Epi epi, char *lds) {
   const int tilesM = int((M + BM - 1) / BM), tilesN = int((N + BN - 1) / BN);
   const int tiles = tilesM * tilesN, workgroups = gridDim.x * gridDim.y;
   for (int id = blockIdx.y * gridDim.x + blockIdx.x; id < tiles; id += workgroups) {
-    gemm_tile<T, kAT, kBT, Epi, kProbe>(A, B, M, N, K, epi, lds, tilesM, tilesN, id);
+    gemm_tile<T, kAT, kBT, Epi, kProbe, kTail>(A, B, M, N, K, epi, lds, tilesM, tilesN, id);
     if (id + workgroups < tiles)
       __syncthreads(); // the ring is reused by this workgroup's next tile
   }
@@ -558,19 +578,21 @@ __device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B,
                                            Epi epi) {
   // 4 stages x (256 + 256) rows x 32 k x 2 B = 128 KiB of the CU's 160 KiB LDS.
   __shared__ __attribute__((aligned(16))) char lds[kStages * kRStage];
-  // The MFMA path wants K in whole 32-wide steps and 16-byte aligned rows in memory: a row of
-  // B [K,N] (or of A [K,M] when transposed) is N (M) elements long, so those must be multiples
-  // of 8.  M and N need not divide the tile: edge tiles multiply padding and store what exists.
+  // The MFMA path wants 16-byte aligned rows in memory: K % 8 == 0 (rows of A [M,K], of B [N,K]), and a
+  // row of B [K,N] (or of A [K,M] when transposed) is N (M) elements long, so those must be multiples
+  // of 8 as well.  K need not fill the last 32-wide step: its copies fetch zeros beyond K.  M and N need not divide the tile: edge tiles multiply padding and store what exists.
   // An operand whose rows are strided in memory is addressed with 32-bit byte offsets from one
   // buffer descriptor, so it has to stay below 2 GiB; a k-contiguous one below 4 Mi elements per row.
   constexpr int64_t kMaxBytes = int64_t(1) << 31, kMaxRow = int64_t(1) << 22;
   const bool fitsA = kAT ? K * M * 2 < kMaxBytes : K < kMaxRow;
   const bool fitsB = kBT ? K < kMaxRow : K * N * 2 < kMaxBytes;
-  const bool tileable = M > 0 && N > 0 && K > 0 && K % RK == 0 && (kBT || N % 8 == 0) && (!kAT || M % 8 == 0) &&
+  const bool tileable = M > 0 && N > 0 && K > 0 && K % 8 == 0 && (kBT || N % 8 == 0) && (!kAT || M % 8 == 0) &&
                         fitsA && fitsB &&
                         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
-  if (tileable)
-    gemm_tiled<T, kAT, kBT, Epi, kProbe>(A, B, M, N, K, epi, lds);
+  if (tileable && K % RK == 0)
+    gemm_tiled<T, kAT, kBT, Epi, kProbe, false>(A, B, M, N, K, epi, lds);
+  else if (tileable)
+    gemm_tiled<T, kAT, kBT, Epi, kProbe, true>(A, B, M, N, K, epi, lds);
   else
     gemm_scalar<T, kAT, kBT, Epi>(A, B, M, N, K, epi);
 }

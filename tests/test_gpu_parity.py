@@ -663,9 +663,9 @@ def test_gemm_golden_3x3(host, orc, stream):
     assert np.all(orc.half_to_float(out) == g["expected_fill"])
 
 
-@pytest.mark.parametrize("M,N,K", [(5, 7, 9), (100, 36, 130), (256, 256, 16), (256, 256, 48), (255, 252, 64), (17, 300, 64)])
+@pytest.mark.parametrize("M,N,K", [(5, 7, 9), (100, 36, 130), (256, 256, 20), (256, 256, 44), (255, 252, 64), (17, 300, 64)])
 def test_gemm_untileable_shapes_bit_exact(host, orc, stream, M, N, K):
-    """K not a multiple of 32 or N not a multiple of 8: the one-lane-per-output path, which
+    """K not a multiple of 8 or N not a multiple of 8: the one-lane-per-output path, which
     accumulates in the oracle's order."""
     a = orc.fill_uniform(M * K, "f16", 1, -1, 1).reshape(M, K)
     b = orc.fill_uniform(K * N, "f16", 2, -1, 1).reshape(K, N)
@@ -698,6 +698,39 @@ def test_gemm_tiled_small_integers_exact(host, orc, stream, dtype, M, N, K):
     b = orc.fill_int(K * N, dtype, 6, -4, 4).reshape(K, N)
     want = orc.to_float(a, dtype).astype(np.int64) @ orc.to_float(b, dtype).astype(np.int64)
     got = host.gemm(stream, a, b, ab_dtype=dtype)
+    assert np.array_equal(got.astype(np.int64), want)
+
+
+@pytest.mark.parametrize("which", ["plain", "ta", "tb", "acc", "mlp"])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 8), (256, 256, 16), (256, 256, 48), (300, 520, 40), (512, 256, 4096 + 24),
+                                   (64, 72, 104), (1000, 264, 72)])
+def test_gemm_partial_last_k_step(host, orc, stream, which, M, N, K):
+    """K a multiple of 8 but not of the 32-wide step: the MFMA path pads the last step with zeros on the
+    way into LDS.  Integer operands give the exact product in any order, so any stale or foreign value
+    that got multiplied in would show; every operand layout and an epilogue with its own loads."""
+    say("gemm partial K step %s %dx%dx%d" % (which, M, N, K))
+    if which == "ta" and M % 8:
+        M = (M + 7) // 8 * 8
+    dtype = "bf16" if which == "mlp" else "f16"
+    a = orc.fill_int(M * K, dtype, 91, -4, 4).reshape(M, K)
+    b = orc.fill_int(K * N, dtype, 92, -4, 4).reshape(K, N)
+    want = orc.to_float(a, dtype).astype(np.int64) @ orc.to_float(b, dtype).astype(np.int64)
+    if which == "plain":
+        got = _gemm_guarded(host, stream, "imex_gemm_f16_f16_f32", a, b, M, N, K)
+    elif which == "ta":
+        got = _gemm_guarded(host, stream, "imex_gemm_f16_f16_f32_ta", np.ascontiguousarray(a.T), b, M, N, K)
+    elif which == "tb":
+        got = _gemm_guarded(host, stream, "imex_gemm_f16_f16_f32_tb", a, np.ascontiguousarray(b.T), M, N, K)
+    elif which == "acc":
+        c0 = orc.fill_int(M * N, "f32", 93, -1000, 1000).reshape(M, N)
+        got = host.gemm(stream, a, b, c=c0, ab_dtype="f16")
+        want = want + c0.astype(np.int64)
+    else:
+        bias = orc.fill_int(N, "f32", 94, -3, 3)
+        out = _gemm_guarded(host, stream, "imex_gemm_bf16_bias_silu_bf16", a, b, M, N, K, extra=(bias,), out_np=np.uint16)
+        ref = orc.bfloat_to_float(orc.bias_silu_bf16(want.astype(np.float32), bias))
+        assert np.max(np.abs(orc.bfloat_to_float(out) - ref)) <= 2.0 ** -7 * np.max(np.abs(ref)) + 1e-6
+        return
     assert np.array_equal(got.astype(np.int64), want)
 
 

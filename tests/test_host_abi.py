@@ -88,7 +88,8 @@ def test_launch_shapes(host):
     assert ls("imex_gemm_f16_f16_f32", [512, 256, 96])[0] == (2, 1, 1)
     assert ls("imex_gemm_f16_f16_f32", [255, 256, 64])[0] == (1, 1, 1)
     assert ls("imex_gemm_f16_f16_f32", [257, 520, 64])[0] == (6, 1, 1)
-    assert ls("imex_gemm_f16_f16_f32", [256, 256, 48])[0] == (128, 1, 1)   # K % 32 != 0: one lane per output
+    assert ls("imex_gemm_f16_f16_f32", [256, 256, 48])[0] == (1, 1, 1)     # K % 32 != 0 but K % 8 == 0: still tiled
+    assert ls("imex_gemm_f16_f16_f32", [256, 256, 44])[0] == (128, 1, 1)   # K % 8 != 0: one lane per output
     assert ls("imex_gemm_f16_f16_f32", [256, 252, 64])[0] == (126, 1, 1)   # N % 8 != 0
     assert ls("imex_gemm_f16_f16_f32_tb", [256, 252, 64])[0] == (1, 1, 1)  # B stored [N,K]: any N
     assert ls("imex_gemm_f16_f16_f32_ta", [252, 256, 64])[0] == (126, 1, 1)  # A stored [K,M]: M % 8 != 0
@@ -323,12 +324,12 @@ def test_launch_shapes_cover_the_problem(host):
            round_k=st.booleans())
     def gemm(M, N, k, round_n, round_k):
         N = (N + 7) // 8 * 8 if round_n else N
-        K = k * 32 if round_k else k * 7 + 5
+        K = k * 8 if round_k else k * 7 + 5
         for name in ("imex_gemm_f16_f16_f32", "imex_gemm_f16_f16_f32_ta", "imex_gemm_f16_f16_f32_tb",
                      "imex_gemm_bf16_bias_silu_bf16"):
             (gx, gy, gz), block, _ = ls(name, [M, N, K])
             assert block == (512, 1, 1) and gy == gz == 1
-            tileable = K % 32 == 0 and (name.endswith("_tb") or N % 8 == 0) and (not name.endswith("_ta") or M % 8 == 0)
+            tileable = K % 8 == 0 and (name.endswith("_tb") or N % 8 == 0) and (not name.endswith("_ta") or M % 8 == 0)
             assert gx == -(-M // 256) * -(-N // 256) if tileable else gx * 512 >= M * N
 
     eltwise()
