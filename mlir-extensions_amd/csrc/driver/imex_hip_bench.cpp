@@ -13,7 +13,7 @@
 // runtime):avg: ..." line per workload, the line bench_imex greps into
 // report.txt (bench_imex.in:87-91).
 //
-//   imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--rotate S] [--launch-only N] <workload>...
+//   imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--rotate S] [--grid G] [--launch-only N] <workload>...
 //   imex-hip-bench --list
 //   imex-hip-bench [-l] --report report.txt <workload>...|all|operators
 //
@@ -27,6 +27,7 @@
 //   --rotate S     S separate copies of the workload's tensors, launches walking round them: with S x footprint
 //                  beyond the 256 MiB Infinity Cache every launch streams from HBM (back-to-back figure and
 //                  --launch-only runs; the per-launch statistics stay on the first set)
+//   --grid G       launch G x 1 x 1 workgroups instead of the catalogue's grid (the kernels stride over their work)
 //   --launch-only  skip the timing loop and just launch the kernel N times (for
 //                  rocprofv3 counter runs, which time and count every dispatch themselves)
 //
@@ -182,6 +183,12 @@ std::vector<Workload> workloads() {
       {"gemm_f16_4096_probe_copies_only", "imex_gemm_probe_copies_only", {},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_f16_4096_probe_copies_only_a", "imex_gemm_probe_copies_only_a", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_f16_4096_probe_copies_only_b", "imex_gemm_probe_copies_only_b", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
       {"mfma_lds_ceiling_f16_every_exponent", "imex_mfma_lds_ceiling_f16", {256 * 512},
        {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 2}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
   };
@@ -221,7 +228,7 @@ std::string programDir() {
 }
 
 struct Options {
-  int runs = 100, warmups = 10, launchOnly = 0, rotate = 1;
+  int runs = 100, warmups = 10, launchOnly = 0, rotate = 1, grid = 0;
   bool flush = false, zeros = false;
 };
 
@@ -266,6 +273,10 @@ int runWorkload(const Workload &w, const Options &opt) {
       return 1;
     }
     blob = imexHipKernelModule(w.kernel, &blobSize);
+  }
+  if (opt.grid > 0) { // every kernel strides over its work, so any grid computes the same thing
+    grid[0] = static_cast<size_t>(opt.grid);
+    grid[1] = grid[2] = 1;
   }
   void *module = gpuModuleLoad(stream, blob, blobSize);
   void *kernel = gpuKernelGet(stream, module, w.kernel);
@@ -422,6 +433,9 @@ int main(int argc, char **argv) {
       childOptions += " --warmups " + std::to_string(opt.warmups);
     } else if (a == "--launch-only" && i + 1 < argc) {
       opt.launchOnly = atoi(argv[++i]);
+    } else if (a == "--grid" && i + 1 < argc) {
+      opt.grid = atoi(argv[++i]);
+      childOptions += " --grid " + std::to_string(opt.grid);
     } else if (a == "--rotate" && i + 1 < argc) {
       opt.rotate = atoi(argv[++i]);
       childOptions += " --rotate " + std::to_string(opt.rotate);
@@ -434,7 +448,7 @@ int main(int argc, char **argv) {
     }
   }
   if (names.empty() || opt.runs < 1 || opt.rotate < 1 || opt.rotate > 64) {
-    fprintf(stderr, "usage: imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--rotate S] [--launch-only N] [--report FILE] <workload>|all ...\n"
+    fprintf(stderr, "usage: imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--rotate S] [--grid G] [--launch-only N] [--report FILE] <workload>|all ...\n"
                     "       imex-hip-bench --list\n");
     return 2;
   }

@@ -69,6 +69,8 @@ enum : int {
   kProbeNoLoopCopies = 1, // no global -> LDS copies inside the K loop (the prologue fills all four ring stages once)
   kProbeNoEpilogue = 2,   // accumulators kept alive but not stored
   kProbeCopiesOnly = 4,   // no LDS fragment reads and no MFMAs: the copy pipeline and its barriers alone
+  kProbeNoCopyA = 8,      // A's slabs are not copied
+  kProbeNoCopyB = 16,     // B's slabs are not copied
 };
 
 // Wavefront grid inside the 256 x 256 workgroup tile: 2 x 4, each wavefront 128 x 64.
@@ -362,8 +364,10 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   constexpr int kImgA = 0, kImgB = kImageBytes;
   auto dma_tile = [&](int kt, int stageOff) { // stageOff: byte offset of the ring stage, wave-uniform
     const bool partial = kTail && kt == lastTile;
-    opA.dma(lds_base, stageOff + kImgA, kt, partial);
-    opB.dma(lds_base, stageOff + kImgB, kt, partial);
+    if constexpr (!(kProbe & kProbeNoCopyA))
+      opA.dma(lds_base, stageOff + kImgA, kt, partial);
+    if constexpr (!(kProbe & kProbeNoCopyB))
+      opB.dma(lds_base, stageOff + kImgB, kt, partial);
   };
 
   // acc[i][j] is the 16 x 16 block at rows 16 i, columns 16 j of the wavefront's tile, held
@@ -463,7 +467,10 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
       dma_tile(min(t + kDist, lastTile), dmaOff);
     IMEX_FENCE();
     half0(p, curOff);                               // rows 0-63 of tile t; reads its rows 64-127
-    wait_vmcnt<(kDist - 1) * 2 * kDmaPerWave>();    // tile t+1 has landed (this wavefront's part) ...
+    if constexpr (kProbe & (kProbeNoCopyA | kProbeNoCopyB))
+      wait_vmcnt<(kDist - 1) * kDmaPerWave>();      // (probe with one operand's copies only)
+    else
+      wait_vmcnt<(kDist - 1) * 2 * kDmaPerWave>();  // tile t+1 has landed (this wavefront's part) ...
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();                   // ... and everyone else's; all reads of tile t are done
     IMEX_FENCE();

@@ -118,3 +118,5 @@ IMEX_GEMM_PROBE(imex_gemm_probe_no_loop_copies, imexhip_gemm::kProbeNoLoopCopies
 IMEX_GEMM_PROBE(imex_gemm_probe_no_epilogue, imexhip_gemm::kProbeNoEpilogue)
 IMEX_GEMM_PROBE(imex_gemm_probe_multiply_only, imexhip_gemm::kProbeNoLoopCopies | imexhip_gemm::kProbeNoEpilogue)
 IMEX_GEMM_PROBE(imex_gemm_probe_copies_only, imexhip_gemm::kProbeCopiesOnly)
+IMEX_GEMM_PROBE(imex_gemm_probe_copies_only_a, imexhip_gemm::kProbeCopiesOnly | imexhip_gemm::kProbeNoCopyB)
+IMEX_GEMM_PROBE(imex_gemm_probe_copies_only_b, imexhip_gemm::kProbeCopiesOnly | imexhip_gemm::kProbeNoCopyA)
