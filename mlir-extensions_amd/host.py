@@ -162,9 +162,18 @@ def launch_shape(kernel, dims):
     return tuple(grid), tuple(block), smem.value
 
 
+_SIGNATURE_TYPES = {}
+
+
 def signature_types(kernel):
     """Argument types of a catalogue kernel, from its signature string
     "(in: f32*, out: f32*, rows: i64, init: f32)" -> ["ptr", "ptr", "i64", "f32"]; None if unknown."""
+    if kernel not in _SIGNATURE_TYPES:
+        _SIGNATURE_TYPES[kernel] = _parse_signature(kernel)
+    return _SIGNATURE_TYPES[kernel]
+
+
+def _parse_signature(kernel):
     k = kernels()
     for i in range(k.imexHipKernelCount()):
         if k.imexHipKernelName(i).decode() == kernel:
