@@ -89,7 +89,12 @@ void *gpuKernelGet(void *queue, void *module, const char *name);
  * stream (a wait on it then waits longer than needed, never shorter).
  * Environment (LevelZeroRuntimeWrappers.cpp:521-597): IMEX_ENABLE_PROFILING,
  * IMEX_PROFILING_RUNS (default 1000), IMEX_PROFILING_WARMUPS (default 3),
- * IMEX_ENABLE_CACHE_FLUSHING, plus IMEX_CACHE_FLUSH_BYTES (default 512 MiB). */
+ * IMEX_ENABLE_CACHE_FLUSHING, plus IMEX_CACHE_FLUSH_BYTES (default 512 MiB:
+ * that many bytes are filled and as many of a second region read before each
+ * timed run, so the caches hold neither the kernel's data nor dirty lines).
+ * Each run's time is the dispatch's own start-to-end interval, as the
+ * reference's is; IMEX_PROFILING_EVENT_PAIRS=1 records events around the
+ * launch instead. */
 void *gpuLaunchKernel(void *queue, void *kernel, size_t gridX, size_t gridY, size_t gridZ,
                       size_t blockX, size_t blockY, size_t blockZ, size_t sharedMemBytes,
                       void *params, void *depEvents);

@@ -29,6 +29,15 @@
 
 #include <hip/hip_runtime_api.h>
 
+// From <hip/hip_ext.h>, which a host compiler cannot include whole: a module launch that attaches a start
+// and a stop event to the dispatch.  Global sizes are in work-items.
+extern "C" hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t globalWorkSizeX, uint32_t globalWorkSizeY,
+                                               uint32_t globalWorkSizeZ, uint32_t localWorkSizeX,
+                                               uint32_t localWorkSizeY, uint32_t localWorkSizeZ,
+                                               size_t sharedMemBytes, hipStream_t hStream, void **kernelParams,
+                                               void **extra, hipEvent_t startEvent, hipEvent_t stopEvent,
+                                               uint32_t flags);
+
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -372,6 +381,12 @@ void enqueue(GpuHipQueue *queue, LaunchArgs &la) {
                                   la.kernelParams.empty() ? nullptr : la.kernelParams.data(), nullptr));
 }
 
+void fillMemory(GpuHipQueue *q, void *dst, unsigned value, size_t count, int bits);
+hipModule_t runtimeModule(GpuHipQueue *q);
+
+// The profiler's cache flush works on a buffer of twice `bytes` (as LevelZeroRuntimeWrappers.cpp:531-538
+// allocates twice the cache size): the first half is filled before every timed launch, the second half,
+// zeroed once here, is then read.
 void ensureFlushBuffer(GpuHipQueue *queue, size_t bytes) {
   if (queue->flushBytes >= bytes)
     return;
@@ -379,8 +394,24 @@ void ensureFlushBuffer(GpuHipQueue *queue, size_t bytes) {
     CHECK_HIP(hipFree(queue->flushBuffer));
   queue->flushBuffer = nullptr;
   queue->flushBytes = 0;
-  CHECK_HIP(hipMalloc(&queue->flushBuffer, bytes));
+  CHECK_HIP(hipMalloc(&queue->flushBuffer, 2 * bytes + 256));
   queue->flushBytes = bytes;
+  fillMemory(queue, queue->flushBuffer, 0, (2 * bytes + 256) / 4, 32);
+}
+
+// Evict the previous run's data (LevelZeroRuntimeWrappers.cpp:524-530,564-570: a cached fill larger than
+// the last-level cache), then read the buffer's other half.  The fill alone leaves the caches full of
+// DIRTY lines, and their write-back would share HBM with the timed kernel; after the read they hold
+// clean lines of a region the kernel does not touch.
+void flushCaches(GpuHipQueue *queue, size_t bytes) {
+  bytes &= ~size_t(15);
+  fillMemory(queue, queue->flushBuffer, 0, bytes / 4, 32);
+  hipFunction_t sweep = getKernel(runtimeModule(queue), "imex_runtime_read_sweep");
+  const void *src = static_cast<const char *>(queue->flushBuffer) + bytes;
+  void *sink = static_cast<char *>(queue->flushBuffer) + 2 * bytes;
+  int64_t vecs = static_cast<int64_t>(bytes / 16);
+  void *params[] = {&src, &vecs, &sink};
+  CHECK_HIP(hipModuleLaunchKernel(sweep, 2048, 1, 1, 256, 1, 1, 0, queue->stream, params, nullptr));
 }
 
 // The profiling loop of LevelZeroRuntimeWrappers.cpp:553-583 on HIP events.
@@ -404,13 +435,28 @@ void profile(GpuHipQueue *queue, LaunchArgs &la, int warmups, int rounds, size_t
     CHECK_HIP(hipEventSynchronize(stop));
     CHECK_HIP(hipEventElapsedTime(&timesMs[0], start, stop));
   } else {
+    // work-item counts of the launch must fit the 32-bit arguments of the launch that takes events
+    bool timestampsOnLaunch = !getenv("IMEX_PROFILING_EVENT_PAIRS");
+    for (int d = 0; d < 3; ++d)
+      timestampsOnLaunch = timestampsOnLaunch && uint64_t(la.grid[d]) * la.block[d] <= 0xffffffffull;
     for (int r = 0; r < rounds; ++r) {
-      // Evict the previous run's data: write a buffer larger than L2 + MALL.
       if (flushBytes)
-        CHECK_HIP(hipMemsetAsync(queue->flushBuffer, 0, flushBytes, queue->stream));
-      CHECK_HIP(hipEventRecord(start, queue->stream));
-      enqueue(queue, la);
-      CHECK_HIP(hipEventRecord(stop, queue->stream));
+        flushCaches(queue, flushBytes);
+      // The reference reads the kernel's own start and end timestamps (command_start / command_end of the
+      // event attached to the launch, LevelZeroRuntimeWrappers.cpp:572-582).  The launch below attaches the
+      // two events to the dispatch in the same way; events recorded around it would add the stream's
+      // bookkeeping between commands to a 10-40 us kernel.
+      if (timestampsOnLaunch) {
+        CHECK_HIP(hipExtModuleLaunchKernel(la.fn, la.grid[0] * la.block[0], la.grid[1] * la.block[1],
+                                           la.grid[2] * la.block[2], la.block[0], la.block[1], la.block[2],
+                                           la.sharedMemBytes, queue->stream,
+                                           la.kernelParams.empty() ? nullptr : la.kernelParams.data(), nullptr,
+                                           start, stop, 0));
+      } else {
+        CHECK_HIP(hipEventRecord(start, queue->stream));
+        enqueue(queue, la);
+        CHECK_HIP(hipEventRecord(stop, queue->stream));
+      }
       CHECK_HIP(hipEventSynchronize(stop));
       CHECK_HIP(hipEventElapsedTime(&timesMs[r], start, stop));
     }
@@ -505,6 +551,10 @@ GpuHipQueue *defaultQueue() {
 // The fill kernels this library carries (csrc/runtime/fill.hip), embedded at build time.
 extern "C" const char imex_runtime_fill_blob[], imex_runtime_fill_blob_end[];
 
+hipModule_t runtimeModule(GpuHipQueue *q) {
+  return loadModule(q, imex_runtime_fill_blob, size_t(imex_runtime_fill_blob_end - imex_runtime_fill_blob));
+}
+
 // `count` elements of `bits` (16 or 32) wide, each set to the low bits of `value`.  A kernel launch, not
 // a memset on the stream: memset nodes recorded into a captured HIP graph have replayed wrongly on this
 // platform, and the queue may sit on a stream its owner captures.
@@ -518,9 +568,7 @@ void fillMemory(GpuHipQueue *q, void *dst, unsigned value, size_t count, int bit
   if (reinterpret_cast<uintptr_t>(dst) % (bits / 8))
     throw std::runtime_error("memset: destination is not aligned to its " + std::to_string(bits) + "-bit elements");
   CHECK_HIP(hipSetDevice(q->device));
-  hipModule_t module =
-      loadModule(q, imex_runtime_fill_blob, size_t(imex_runtime_fill_blob_end - imex_runtime_fill_blob));
-  hipFunction_t fill = getKernel(module, bits == 32 ? "imex_runtime_fill_b32" : "imex_runtime_fill_b16");
+  hipFunction_t fill = getKernel(runtimeModule(q), bits == 32 ? "imex_runtime_fill_b32" : "imex_runtime_fill_b16");
   uint32_t word = value;
   int64_t n = static_cast<int64_t>(count);
   void *params[] = {&dst, &word, &n};
