@@ -130,6 +130,25 @@ def test_profile_helper_modes(host, orc, stream):
     stream.free(d_out)
 
 
+def test_profiled_launch_runs_the_whole_grid(host, orc, stream):
+    """The profiler's timed launches attach their timestamps to the dispatch through a launch call that
+    takes sizes in work-items, not workgroups: a launch with a two-dimensional grid must still cover the
+    whole problem, flushed or not."""
+    zh, n_ctx = 3, 512
+    q, k, v = (orc.fill_uniform(zh * n_ctx * 64, "f16", 70 + i, -1, 1).reshape(zh * n_ctx, 64) for i in range(3))
+    expected = host.flash_attention(stream, q, k, v, zh, n_ctx, 0.125)
+    d_q, d_k, d_v = stream.to_device(q), stream.to_device(k), stream.to_device(v)
+    d_o = stream.alloc(q.size * 2)
+    for flush_bytes in (0, 16 << 20):
+        stream.memset(d_o, 0x7e00, q.size, 16)
+        times = stream.profile("imex_flash_attention_fwd_f16", [zh, n_ctx], [d_q, d_k, d_v, d_o, 0.125, zh, n_ctx],
+                               warmups=0, rounds=2, flush_bytes=flush_bytes, mode=0)
+        assert len(times) == 2 and all(0 < t < 50 for t in times)
+        assert np.array_equal(stream.from_device(d_o, q.shape, np.uint16), expected)
+    for p in (d_q, d_k, d_v, d_o):
+        stream.free(p)
+
+
 def test_profiling_env_prints_reference_line():
     prog = ("import sys; sys.path.insert(0, %r)\nimport __graft_entry__ as e\nimport numpy as np\n"
             "host = e.load_package().host\ns = host.Stream()\n"
