@@ -21,7 +21,8 @@
 //             input fusion (a, b, out, rows: i64, cols: i64) dims = {rows, cols}
 // Launch: block (256,1,1); loop fusion grid ceil(n / 4096) (f32) or ceil(n / 8192)
 // (16-bit), a quarter of that per workgroup below 4 Mi elements; input fusion grid ceil(cols / c), a workgroup per block of c = 64 .. 4 columns
-// (the widest that leaves 512 workgroups).  Workgroups stride, so any grid is correct.
+// (the widest that leaves 512 workgroups), or, from 2048 rows and 128 row segments of 128 bytes on, block
+// (576,1,1) and grid ceil(cols * element bytes / 128): the streaming form.  Workgroups stride, so any grid is correct.
 
 #include "device_common.h"
 
@@ -197,6 +198,35 @@ __device__ __forceinline__ void loop_fusion(const void *__restrict__ a, const vo
 // there is a next tile to overlap with; tall ones are faster with fewer barriers.
 constexpr int kTileElems = 4096, kSmallTileElems = 1024;
 
+// acc + t[0] + t[stride] + ... + t[(n-1) stride], added in that order: sixteen LDS reads are in flight
+// while the previous sixteen values are added.
+__device__ __forceinline__ float add_in_row_order(float acc, const float *t, int n, int stride) {
+  float v[16], w[16];
+  int r = 0;
+  if (n >= 16) {
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      v[u] = t[u * stride];
+    for (r = 16; r + 16 <= n; r += 16) {
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        w[u] = t[(r + u) * stride];
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        acc = acc + v[u];
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        v[u] = w[u];
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      acc = acc + v[u];
+  }
+  for (; r < n; ++r)
+    acc = acc + t[r * stride];
+  return acc;
+}
+
 template <Dt D, int kCols, int kTileElems = ::kTileElems>
 __device__ __forceinline__ void input_fusion_cols(const void *__restrict__ a, const void *__restrict__ b,
                                                   void *__restrict__ out, int64_t rows, int64_t cols,
@@ -205,6 +235,7 @@ __device__ __forceinline__ void input_fusion_cols(const void *__restrict__ a, co
   constexpr int kTileRows = kTileElems / kCols;
   constexpr int kPerLane = kTileElems / kThreads;
   const int tid = threadIdx.x;
+  const bool worker = tid < kThreads; // a launch with more lanes: the others only take part in the barriers
   for (int64_t c0 = int64_t(blockIdx.x) * kCols; c0 < cols; c0 += int64_t(gridDim.x) * kCols) {
     float acc = 0.0f;
     int buf = 0;
@@ -215,7 +246,7 @@ __device__ __forceinline__ void input_fusion_cols(const void *__restrict__ a, co
       for (int u = 0; u < kPerLane; ++u) {
         const int e = u * kThreads + tid;
         const int64_t r = r0 + e / kCols, c = c0 + e % kCols;
-        const bool ok = r < rows && c < cols;
+        const bool ok = worker && r < rows && c < cols;
         xa[u] = ok ? E::get(a, r * cols + c) : 2.0f; // positions outside the matrix: any ordinary value, never added
         xb[u] = ok ? E::get(b, r * cols + c) : 2.0f;
       }
@@ -226,46 +257,129 @@ __device__ __forceinline__ void input_fusion_cols(const void *__restrict__ a, co
       if (__builtin_amdgcn_ballot_w64(!ordinary) == 0) { // uniform over the wavefront
 #pragma unroll
         for (int u = 0; u < kPerLane; ++u)
-          if (r0 + (u * kThreads) / kCols < rows) // uniform: passes that lie wholly below the last row are skipped
+          if (worker && r0 + (u * kThreads) / kCols < rows) // passes that lie wholly below the last row are skipped
             t[u * kThreads + tid] = input_chain<true>(xa[u], xb[u], table);
       } else {
 #pragma unroll
         for (int u = 0; u < kPerLane; ++u)
-          if (r0 + (u * kThreads) / kCols < rows)
+          if (worker && r0 + (u * kThreads) / kCols < rows)
             t[u * kThreads + tid] = input_chain(xa[u], xb[u], table);
       }
       __syncthreads(); // the tile is complete; the other buffer was consumed before the previous barrier
       if (tid < kCols && c0 + tid < cols) {
         const int n = rows - r0 < kTileRows ? int(rows - r0) : kTileRows;
-        // sixteen LDS reads are in flight while the previous sixteen values are added in row order
-        float v[16], w[16];
-        int r = 0;
-        if (n >= 16) {
-#pragma unroll
-          for (int u = 0; u < 16; ++u)
-            v[u] = t[u * kCols + tid];
-          for (r = 16; r + 16 <= n; r += 16) {
-#pragma unroll
-            for (int u = 0; u < 16; ++u)
-              w[u] = t[(r + u) * kCols + tid];
-#pragma unroll
-            for (int u = 0; u < 16; ++u)
-              acc = acc + v[u];
-#pragma unroll
-            for (int u = 0; u < 16; ++u)
-              v[u] = w[u];
-          }
-#pragma unroll
-          for (int u = 0; u < 16; ++u)
-            acc = acc + v[u];
-        }
-        for (; r < n; ++r)
-          acc = acc + t[r * kCols + tid];
+        acc = add_in_row_order(acc, t + tid, n, kCols);
       }
     }
     if (tid < kCols && c0 + tid < cols)
       E::put(out, c0 + tid, acc);
     __syncthreads(); // both buffers are free for the next block of columns
+  }
+}
+
+// ---- kInputFusion on tall, wide matrices: the streaming form --------------------------------
+// With 4 .. 64 columns per workgroup the form above reads 16 .. 64-byte row segments, computes and adds
+// in turn, and is bound by memory latency (17 % of HBM at 8192 x 8192).  Here a workgroup of 576 lanes
+// owns the columns of one 128-byte row segment (32 f32 or 64 16-bit columns).  Its first 512 lanes are
+// workers: 16 bytes per lane and access, 8 lanes per row, 64 rows per access; a tile is 8192 elements
+// (256 or 128 rows), the next tile's loads are issued before this tile's chains are evaluated, and the
+// results go into one of two LDS tiles.  The ninth wavefront does nothing but the ordered additions, one
+// lane per column, a tile behind the workers: one barrier per tile, passed by everybody, hands a tile
+// over and returns the other one.
+constexpr int kStreamWorkers = 512, kStreamThreads = kStreamWorkers + 64;
+constexpr int kStreamTileElems = 8192;
+constexpr int64_t kStreamFromRows = 2048;
+
+template <Dt D> struct StreamShape {
+  static constexpr int kCols = 128 / Elem<D>::kBytes;           // columns per workgroup
+  static constexpr int kRowsPerPass = kStreamWorkers / 8;       // 64
+  static constexpr int kTileRows = kStreamTileElems / kCols;    // 256 (f32) or 128 (16-bit)
+  static constexpr int kPasses = kTileRows / kRowsPerPass;      // 4 or 2
+};
+
+// what the launch and the kernel both decide on: enough column blocks for the chip, enough rows for a pipeline
+template <Dt D> __device__ __forceinline__ bool input_fusion_streams(int64_t rows, int64_t cols) {
+  return rows >= kStreamFromRows && cols >= int64_t(StreamShape<D>::kCols) * 128;
+}
+
+template <Dt D>
+__device__ __forceinline__ void input_fusion_stream(const void *__restrict__ a, const void *__restrict__ b,
+                                                    void *__restrict__ out, int64_t rows, int64_t cols,
+                                                    const LogfEntry *table, float *tile) {
+  using E = Elem<D>;
+  using S = StreamShape<D>;
+  constexpr int kCols = S::kCols, kTileRows = S::kTileRows, kPasses = S::kPasses;
+  const int tid = threadIdx.x;
+  const int64_t tiles = (rows + kTileRows - 1) / kTileRows;
+  for (int64_t c0 = int64_t(blockIdx.x) * kCols; c0 < cols; c0 += int64_t(gridDim.x) * kCols) {
+    if (tid < kStreamWorkers) {
+      const int lr = tid >> 3, lc = (tid & 7) * E::kPerVec; // row within an access, first column of the lane's vector
+      const bool colOk = c0 + lc < cols;                    // cols is a multiple of the vector: all of it or none
+      const char *pa = static_cast<const char *>(a) + (c0 + lc) * E::kBytes;
+      const char *pb = static_cast<const char *>(b) + (c0 + lc) * E::kBytes;
+      // positions outside the matrix: any ordinary value (2.0 in all three types), never added
+      const uint32_t two = D == Dt::F32 ? 0x40000000u : 0x40004000u;
+      u32x4 ca[kPasses], cb[kPasses], na[kPasses], nb[kPasses];
+      auto load_tile = [&](int64_t t, u32x4(&va)[kPasses], u32x4(&vb)[kPasses]) {
+#pragma unroll
+        for (int p = 0; p < kPasses; ++p) {
+          const int64_t r = t * kTileRows + p * S::kRowsPerPass + lr;
+          va[p] = vb[p] = u32x4{two, two, two, two};
+          if (colOk && r < rows) {
+            va[p] = load128<true>(reinterpret_cast<const u32x4 *>(pa + r * cols * E::kBytes));
+            vb[p] = load128<true>(reinterpret_cast<const u32x4 *>(pb + r * cols * E::kBytes));
+          }
+        }
+      };
+      load_tile(0, ca, cb);
+      for (int64_t t = 0; t < tiles; ++t) {
+        if (t + 1 < tiles)
+          load_tile(t + 1, na, nb);
+        float *dst = tile + (t & 1) * kStreamTileElems + lr * kCols + lc;
+#pragma unroll
+        for (int p = 0; p < kPasses; ++p) {
+          float fa[E::kPerVec], fb[E::kPerVec];
+          E::unpack(ca[p], fa);
+          E::unpack(cb[p], fb);
+          bool ordinary = true;
+#pragma unroll
+          for (int i = 0; i < E::kPerVec; ++i)
+            ordinary = ordinary && logf_ordinary(fb[i]);
+          if (__builtin_amdgcn_ballot_w64(!ordinary) == 0) { // uniform over the wavefront
+#pragma unroll
+            for (int i = 0; i < E::kPerVec; ++i)
+              fa[i] = input_chain<true>(fa[i], fb[i], table);
+          } else {
+#pragma unroll
+            for (int i = 0; i < E::kPerVec; ++i)
+              fa[i] = input_chain(fa[i], fb[i], table);
+          }
+          u32x4 *d = reinterpret_cast<u32x4 *>(dst + p * S::kRowsPerPass * kCols);
+#pragma unroll
+          for (int i = 0; i < E::kPerVec / 4; ++i)
+            d[i] = u32x4{f2u(fa[4 * i]), f2u(fa[4 * i + 1]), f2u(fa[4 * i + 2]), f2u(fa[4 * i + 3])};
+        }
+        __syncthreads(); // tile t is complete; the adder is done with tile t-1, whose buffer tile t+1 goes into
+#pragma unroll
+        for (int p = 0; p < kPasses; ++p) {
+          ca[p] = na[p];
+          cb[p] = nb[p];
+        }
+      }
+    } else {
+      const int col = tid - kStreamWorkers;
+      const bool active = col < kCols && c0 + col < cols;
+      float acc = 0.0f;
+      for (int64_t t = 0; t < tiles; ++t) {
+        __syncthreads(); // tile t is complete
+        const int n = rows - t * kTileRows < kTileRows ? int(rows - t * kTileRows) : kTileRows;
+        if (active)
+          acc = add_in_row_order(acc, tile + (t & 1) * kStreamTileElems + col, n, kCols);
+      }
+      if (active)
+        E::put(out, c0 + col, acc);
+    }
+    __syncthreads(); // both tiles are free for the next block of columns
   }
 }
 
@@ -279,8 +393,15 @@ template <Dt D>
 __device__ __forceinline__ void input_fusion(const void *__restrict__ a, const void *__restrict__ b,
                                              void *__restrict__ out, int64_t rows, int64_t cols) {
   __shared__ LogfEntry table[16];
-  __shared__ float tile[2 * kTileElems];
+  __shared__ __attribute__((aligned(16))) float tile[2 * kStreamTileElems];
   stage_table(table);
+  // The launch says which form: 576 lanes ask for the streaming one, which needs whole aligned vectors.
+  const bool vectors = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0 &&
+                       cols % Elem<D>::kPerVec == 0;
+  if (blockDim.x == kStreamThreads && vectors && input_fusion_streams<D>(rows, cols)) {
+    input_fusion_stream<D>(a, b, out, rows, cols, table, tile);
+    return;
+  }
   switch (input_fusion_block_cols(cols)) {
   case 64: input_fusion_cols<D, 64>(a, b, out, rows, cols, table, tile); break;
   case 32: input_fusion_cols<D, 32>(a, b, out, rows, cols, table, tile); break;
@@ -302,7 +423,7 @@ __device__ __forceinline__ void input_fusion(const void *__restrict__ a, const v
       const CTYPE *a, const CTYPE *b, CTYPE *out, int64_t n) {                                                       \
     loop_fusion<DT>(a, b, out, n);                                                                                   \
   }                                                                                                                  \
-  extern "C" __global__ __launch_bounds__(kThreads) void imex_input_fusion_##SUFFIX(                                 \
+  extern "C" __global__ __launch_bounds__(kStreamThreads) void imex_input_fusion_##SUFFIX(                                 \
       const CTYPE *a, const CTYPE *b, CTYPE *out, int64_t rows, int64_t cols) {                                      \
     input_fusion<DT>(a, b, out, rows, cols);                                                                         \
   }

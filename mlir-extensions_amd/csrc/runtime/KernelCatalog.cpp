@@ -27,7 +27,7 @@ extern const unsigned char imex_blob_attention[], imex_blob_attention_end[];
 namespace {
 
 enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm, Fusion, Attention };
-enum class Shape { Eltwise32, Eltwise16, Fusion32, Fusion16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, ReduceOuter16, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, Attention };
+enum class Shape { Eltwise32, Eltwise16, Fusion32, Fusion16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, ReduceOuter16, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, ColumnThreads16, Attention };
 
 struct Entry {
   const char *name;
@@ -69,9 +69,9 @@ const Entry kEntries[] = {
     {"imex_input_fusion_f32", "(a: f32*, b: f32*, out: f32*, rows: i64, cols: i64)", Module::Fusion,
      Shape::ColumnThreads, 2},
     {"imex_input_fusion_f16", "(a: f16*, b: f16*, out: f16*, rows: i64, cols: i64)", Module::Fusion,
-     Shape::ColumnThreads, 2},
+     Shape::ColumnThreads16, 2},
     {"imex_input_fusion_bf16", "(a: bf16*, b: bf16*, out: bf16*, rows: i64, cols: i64)", Module::Fusion,
-     Shape::ColumnThreads, 2},
+     Shape::ColumnThreads16, 2},
     {"imex_flash_attention_fwd_f16",
      "(Q: f16*, K: f16*, V: f16*, Out: f16*, sm_scale: f32, ZH: i64, N_CTX: i64)", Module::Attention,
      Shape::Attention, 2},
@@ -230,8 +230,19 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     }
     break;
   }
-  case Shape::ColumnThreads: { // a workgroup per block of 64 .. 4 columns: the widest that leaves 512 workgroups
-    const int64_t cols = dims[1];
+  case Shape::ColumnThreads:
+  case Shape::ColumnThreads16: {
+    const int64_t rows = dims[0], cols = dims[1];
+    // From 2048 rows and 128 row segments of 128 bytes on: the streaming form, 576 lanes per segment's
+    // columns (32 f32 or 64 16-bit ones).  The kernel applies the same rule, and falls back by itself when
+    // the rows are not made of whole aligned 16-byte vectors.
+    const int64_t segment_cols = e->shape == Shape::ColumnThreads ? 32 : 64;
+    if (rows >= 2048 && cols >= segment_cols * 128) {
+      block[0] = 576;
+      grid[0] = ceilDiv(cols, segment_cols);
+      break;
+    }
+    // otherwise a workgroup per block of 64 .. 4 columns: the widest that leaves 512 workgroups
     const int64_t block_cols = cols >= 64 * 512 ? 64 : cols >= 32 * 512 ? 32 : cols >= 16 * 512 ? 16 : cols >= 8 * 512 ? 8 : 4;
     grid[0] = ceilDiv(cols, block_cols);
     break;

@@ -110,6 +110,12 @@ def test_launch_shapes(host):
     assert ls("imex_flash_attention_fwd_f16", [3, 256])[0] == (4, 3, 1)
     assert ls("imex_input_fusion_f32", [512, 1024])[0] == (256, 1, 1)      # 4 columns per workgroup
     assert ls("imex_input_fusion_f32", [512, 65536])[0] == (1024, 1, 1)    # 64
+    # tall and wide: the streaming form, 576 lanes per 128-byte row segment
+    assert ls("imex_input_fusion_f32", [8192, 8192])[:2] == ((256, 1, 1), (576, 1, 1))
+    assert ls("imex_input_fusion_bf16", [8192, 8192])[:2] == ((128, 1, 1), (576, 1, 1))
+    assert ls("imex_input_fusion_f16", [2048, 8200])[:2] == ((129, 1, 1), (576, 1, 1))
+    assert ls("imex_input_fusion_f32", [2047, 8192])[1] == (256, 1, 1)
+    assert ls("imex_input_fusion_f16", [8192, 4096])[1] == (256, 1, 1)
     assert ls("imex_gemm_4kx4kx4k_transpose_a", []) == ((16, 16, 1), (512, 1, 1), 0)
     assert ls("imex_gemm_f16_f16_f32_tb", [512, 256, 96])[0] == (2, 1, 1)
     with pytest.raises(ValueError):
