@@ -314,27 +314,24 @@ __device__ __forceinline__ void input_fusion_stream(const void *__restrict__ a, 
   for (int64_t c0 = int64_t(blockIdx.x) * kCols; c0 < cols; c0 += int64_t(gridDim.x) * kCols) {
     if (tid < kStreamWorkers) {
       const int lr = tid >> 3, lc = (tid & 7) * E::kPerVec; // row within an access, first column of the lane's vector
-      const bool colOk = c0 + lc < cols;                    // cols is a multiple of the vector: all of it or none
-      const char *pa = static_cast<const char *>(a) + (c0 + lc) * E::kBytes;
-      const char *pb = static_cast<const char *>(b) + (c0 + lc) * E::kBytes;
-      // positions outside the matrix: any ordinary value (2.0 in all three types), never added
-      const uint32_t two = D == Dt::F32 ? 0x40000000u : 0x40004000u;
+      // Rows past the end and, in a partial last block, columns past the end re-read a position inside the
+      // matrix instead (their results are never added): the loads are then unconditional, straight-line
+      // code, and the wait for a tile's data leaves the next tile's loads in flight.
+      const int64_t colOff = c0 + lc < cols ? c0 + lc : c0; // cols is a multiple of the vector: all of it or none
+      const char *pa = static_cast<const char *>(a) + colOff * E::kBytes;
+      const char *pb = static_cast<const char *>(b) + colOff * E::kBytes;
       u32x4 ca[kPasses], cb[kPasses], na[kPasses], nb[kPasses];
       auto load_tile = [&](int64_t t, u32x4(&va)[kPasses], u32x4(&vb)[kPasses]) {
 #pragma unroll
         for (int p = 0; p < kPasses; ++p) {
-          const int64_t r = t * kTileRows + p * S::kRowsPerPass + lr;
-          va[p] = vb[p] = u32x4{two, two, two, two};
-          if (colOk && r < rows) {
-            va[p] = load128<true>(reinterpret_cast<const u32x4 *>(pa + r * cols * E::kBytes));
-            vb[p] = load128<true>(reinterpret_cast<const u32x4 *>(pb + r * cols * E::kBytes));
-          }
+          const int64_t r = min(t * kTileRows + p * S::kRowsPerPass + lr, rows - 1);
+          va[p] = load128<true>(reinterpret_cast<const u32x4 *>(pa + r * cols * E::kBytes));
+          vb[p] = load128<true>(reinterpret_cast<const u32x4 *>(pb + r * cols * E::kBytes));
         }
       };
       load_tile(0, ca, cb);
       for (int64_t t = 0; t < tiles; ++t) {
-        if (t + 1 < tiles)
-          load_tile(t + 1, na, nb);
+        load_tile(t + 1 < tiles ? t + 1 : t, na, nb); // past the last tile: the last one again, unused
         float *dst = tile + (t & 1) * kStreamTileElems + lr * kCols + lc;
 #pragma unroll
         for (int p = 0; p < kPasses; ++p) {
