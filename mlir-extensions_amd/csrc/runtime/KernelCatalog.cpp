@@ -10,6 +10,7 @@
 
 #include "imex_hip_kernels.h"
 
+#include <algorithm>
 #include <cstring>
 
 // Blob symbols come from the assembler stub generated at build time
@@ -208,6 +209,18 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
       grid[1] = 65535;
     if (grid[2] > 65535)
       grid[2] = 65535;
+    // 32-bit problems made of whole 128 x 128 tiles: 512 workgroups (two per CU), each of which walks its
+    // share of the tiles with the next tile's loads in flight while the current one is written
+    if (is32 && big && rows % 128 == 0 && cols % 128 == 0) {
+      const size_t budget = 512;
+      if (grid[0] >= budget) {
+        grid[0] = budget;
+        grid[1] = grid[2] = 1;
+      } else {
+        grid[1] = std::min(grid[1], std::max<size_t>(1, budget / grid[0]));
+        grid[2] = std::min(grid[2], std::max<size_t>(1, budget / (grid[0] * grid[1])));
+      }
+    }
     break;
   }
   case Shape::Attention: {

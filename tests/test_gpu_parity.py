@@ -397,13 +397,29 @@ def test_transpose_large_tiles_ragged(host, orc, stream, rows, cols, dtype):
     assert np.array_equal(got, x.T)
 
 
+@pytest.mark.parametrize("rows,cols", [(4096, 4224), (128, 131072), (8192, 4096)])
+def test_transpose_b32_whole_tiles_pipelined(host, orc, stream, rows, cols):
+    """32-bit problems made of whole 128 x 128 tiles: at most 512 workgroups, each walking two or more tiles
+    with the next tile's loads issued before the current tile is written (an odd and an even number of tiles
+    per workgroup, a single tile row)."""
+    x = np.arange(rows * cols, dtype=np.uint32).reshape(rows, cols)
+    assert np.array_equal(host.transpose2d(stream, x), x.T)
+
+
+def test_transpose3d_b32_whole_tiles_pipelined(host, orc, stream):
+    shape = (256, 64, 1024)
+    x = np.arange(int(np.prod(shape)), dtype=np.uint32).reshape(shape)
+    assert np.array_equal(host.transpose3d(stream, x), x.transpose(2, 1, 0))
+
+
 def test_transpose_any_grid(host, orc, stream):
     """Workgroups stride over the tiles: a grid smaller or larger than one workgroup
     per tile gives the same result."""
     import ctypes as C
-    for name, np_t, rows, cols in [("imex_transpose2d_b32", np.uint32, 4096, 4104), ("imex_transpose2d_b16", np.uint16, 520, 264)]:
+    for name, np_t, rows, cols in [("imex_transpose2d_b32", np.uint32, 4096, 4104), ("imex_transpose2d_b16", np.uint16, 520, 264),
+                                   ("imex_transpose2d_b32", np.uint32, 4096, 4096)]:
         x = np.arange(rows * cols, dtype=np.uint64).astype(np_t).reshape(rows, cols)
-        for grid in [(3, 1, 1), (7, 5, 2)]:
+        for grid in [(3, 1, 1), (7, 5, 2), (40, 30, 1)]:
             d_in, d_out = stream.to_device(x), stream.alloc(x.nbytes)
             fn = stream.kernel(name)
             descs, keep = host._pack_params([d_in, d_out, rows, cols])

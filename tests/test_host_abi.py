@@ -75,7 +75,11 @@ def test_launch_shapes(host):
     assert ls("imex_reduce_outer_f32", [32, 5000])[0] == (5, 1, 1)                  # 1024
     assert ls("imex_transpose2d_b16", [8192, 8192])[0] == (32, 32, 1)   # 256 x 256 tiles from 2^24 elements
     assert ls("imex_transpose2d_b16", [2048, 2048])[0] == (16, 16, 1)   # 128 x 128 below
-    assert ls("imex_transpose2d_b32", [4096, 4096])[0] == (32, 32, 1)   # 128 x 128 tiles from 2^24 elements
+    # 128 x 128 tiles from 2^24 elements; whole tiles: 512 workgroups walk them, the next tile's loads in flight
+    assert ls("imex_transpose2d_b32", [4096, 4096])[0] == (32, 16, 1)
+    assert ls("imex_transpose2d_b32", [4096, 4100])[0] == (33, 32, 1)   # ragged: one workgroup per tile
+    assert ls("imex_transpose2d_b32", [128, 131072])[0] == (512, 1, 1)
+    assert ls("imex_transpose3d_b32", [256, 64, 1024])[0] == (8, 2, 32)
     assert ls("imex_transpose2d_b32", [2048, 4096])[0] == (64, 32, 1)   # 64 x 64 below
     assert ls("imex_transpose2d_b32", [10, 20])[0] == (1, 1, 1)
     assert ls("imex_transpose3d_b32", [16, 96, 96])[0] == (2, 1, 96)
