@@ -125,8 +125,8 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_rowmean_f32(const fl
 // workgroup reads kVecs * 4 KiB contiguous bytes of every slice.  With `outer` slices a power-of-two
 // number of bytes apart, all of a lane's loads fall into the same DRAM channel; wide contiguous
 // spans per workgroup are what keeps the channels streaming (measured on 32 x 4 Mi: 111 us with
-// 4 KiB spans, 83 us with 32 KiB).  Loads of four slices are issued together, adds kept in slice
-// order.  Workgroups stride over the blocks of outputs, so any grid covers everything.
+// 4 KiB spans, 83 us with 32 KiB).  Four slices' loads are kept in flight (a register ring), adds
+// kept in slice order.  Workgroups stride over the blocks of outputs, so any grid covers everything.
 template <io::Dt D, int kVecs>
 __device__ __forceinline__ void reduce_outer_vec(const void *__restrict__ in, void *__restrict__ out, int64_t outer,
                                                  int64_t inner, float init) {
@@ -143,7 +143,6 @@ __device__ __forceinline__ void reduce_outer_vec(const void *__restrict__ in, vo
 #pragma unroll
       for (int e = 0; e < kPer; ++e)
         acc[v][e] = init;
-    const u32x4 zero = {0u, 0u, 0u, 0u};
     auto add = [&](int v, u32x4 raw) {
       float f[kPer];
       E::unpack(raw, f);
@@ -151,29 +150,47 @@ __device__ __forceinline__ void reduce_outer_vec(const void *__restrict__ in, vo
       for (int e = 0; e < kPer; ++e)
         acc[v][e] = acc[v][e] + f[e];
     };
+    // Lanes past the end of the last block read the last vector instead (and store nothing): the loads
+    // are unconditional, so the wait for one slice leaves the loads of the next three in flight.
+    int64_t at[kVecs];
+#pragma unroll
+    for (int v = 0; v < kVecs; ++v) {
+      const int64_t i = i0 + v * (kThreads * kPer);
+      at[v] = (i < inner ? i : inner - kPer) / kPer;
+    }
+    // A ring of four slices: slice o is added, in slice order, and its registers are at once reloaded with
+    // slice o + 4, so three to four slices' loads are in flight all the time.
+    constexpr int kRing = 4;
     int64_t o = 0;
-    for (; o + 4 <= outer; o += 4) {
-      u32x4 t[4][kVecs];
+    if (outer >= kRing) {
+      u32x4 t[kRing][kVecs];
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < kRing; ++u)
 #pragma unroll
-        for (int v = 0; v < kVecs; ++v) {
-          const int64_t i = i0 + v * (kThreads * kPer);
-          t[u][v] = i < inner ? __builtin_nontemporal_load(src + i / kPer + (o + u) * strideVecs) : zero;
+        for (int v = 0; v < kVecs; ++v)
+          t[u][v] = __builtin_nontemporal_load(src + at[v] + u * strideVecs);
+      for (; o + 2 * kRing <= outer; o += kRing) {
+#pragma unroll
+        for (int u = 0; u < kRing; ++u) {
+#pragma unroll
+          for (int v = 0; v < kVecs; ++v)
+            add(v, t[u][v]);
+#pragma unroll
+          for (int v = 0; v < kVecs; ++v)
+            t[u][v] = __builtin_nontemporal_load(src + at[v] + (o + kRing + u) * strideVecs);
         }
+      }
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < kRing; ++u)
 #pragma unroll
         for (int v = 0; v < kVecs; ++v)
           add(v, t[u][v]);
+      o += kRing;
     }
     for (; o < outer; ++o)
 #pragma unroll
-      for (int v = 0; v < kVecs; ++v) {
-        const int64_t i = i0 + v * (kThreads * kPer);
-        if (i < inner)
-          add(v, __builtin_nontemporal_load(src + i / kPer + o * strideVecs));
-      }
+      for (int v = 0; v < kVecs; ++v)
+        add(v, __builtin_nontemporal_load(src + at[v] + o * strideVecs));
 #pragma unroll
     for (int v = 0; v < kVecs; ++v) {
       const int64_t i = i0 + v * (kThreads * kPer);
