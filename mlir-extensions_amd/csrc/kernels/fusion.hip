@@ -286,92 +286,188 @@ __device__ __forceinline__ void input_fusion_cols(const void *__restrict__ a, co
 // results go into one of two LDS tiles.  The ninth wavefront does nothing but the ordered additions, one
 // lane per column, a tile behind the workers: one barrier per tile, passed by everybody, hands a tile
 // over and returns the other one.
+// The same structure serves narrow matrices (fewer than 4096 columns, the reference's 512 x 1024 among them):
+// 256 workers + the adder wavefront = 320 lanes own 4 columns, one element per lane and access, 64 rows per
+// tile, eight tiles' loads in flight together.  There the ordered additions are the critical path
+// (a lone wavefront issues a dependent addition every ~8 cycles), and what this form buys is that nothing
+// else is ever on it: the adder never loads or evaluates, and the workers are always a tile ahead.
 constexpr int kStreamWorkers = 512, kStreamThreads = kStreamWorkers + 64;
+constexpr int kNarrowWorkers = 256, kNarrowThreads = kNarrowWorkers + 64;
 constexpr int kStreamTileElems = 8192;
+constexpr int kStreamTileFloats = 64 * (128 + 4); // the largest padded tile: 64 columns of 128 rows
 constexpr int64_t kStreamFromRows = 2048;
 
-template <Dt D> struct StreamShape {
-  static constexpr int kCols = 128 / Elem<D>::kBytes;           // columns per workgroup
-  static constexpr int kRowsPerPass = kStreamWorkers / 8;       // 64
-  static constexpr int kTileRows = kStreamTileElems / kCols;    // 256 (f32) or 128 (16-bit)
-  static constexpr int kPasses = kTileRows / kRowsPerPass;      // 4 or 2
+// kLanesPerRow worker lanes cover a row segment, each with one 16-byte vector (kVec) or one element; an access
+// of all workers is a pass, kTilePasses passes make a tile (what is handed to the adder at one barrier), and
+// the loads of kGroupTiles tiles are issued together, one such group ahead of the one being evaluated.
+template <Dt D, int kLanesPerRow, int kWorkers, int kTilePassesT, int kGroupTilesT, bool kVecT> struct StreamShape {
+  static constexpr bool kVec = kVecT;
+  static constexpr int kLanes = kLanesPerRow, kWork = kWorkers, kTilePasses = kTilePassesT, kGroupTiles = kGroupTilesT;
+  static constexpr int kPer = kVec ? Elem<D>::kPerVec : 1;      // elements per lane and access
+  static constexpr int kCols = kLanesPerRow * kPer;             // columns per workgroup
+  static constexpr int kRowsPerPass = kWorkers / kLanesPerRow;
+  static constexpr int kTileRows = kTilePasses * kRowsPerPass;
+  static constexpr int kGroupPasses = kTilePasses * kGroupTiles;
+  // A tile lies in LDS COLUMN by column, kTileRows + 4 floats apart: the adder reads four consecutive rows of its
+  // column with one 128-bit access, and the pad puts the columns of neighbouring lanes into different banks.
+  static constexpr int kColPitch = kTileRows + 4;
+  static constexpr int kTileFloats = kCols * kColPitch;
+  static_assert(kTileRows % 32 == 0 && kTileFloats <= kStreamTileFloats, "the LDS tiles are sized for 8448 floats");
 };
+// wide: 128-byte row segments, 8192-element tiles (256 rows of 32 f32, 128 rows of 64 16-bit columns)
+template <Dt D>
+using WideShape = StreamShape<D, 8, kStreamWorkers, kStreamTileElems / (128 / Elem<D>::kBytes) / (kStreamWorkers / 8), 1, true>;
+// narrow: four columns, one element per lane, 64 rows per tile (a lane's first result is ready after ONE chain),
+// the loads of eight tiles -- 512 rows -- in flight together
+template <Dt D> using NarrowShape = StreamShape<D, 4, kNarrowWorkers, 1, 8, false>;
 
 // what the launch and the kernel both decide on: enough column blocks for the chip, enough rows for a pipeline
 template <Dt D> __device__ __forceinline__ bool input_fusion_streams(int64_t rows, int64_t cols) {
-  return rows >= kStreamFromRows && cols >= int64_t(StreamShape<D>::kCols) * 128;
+  return rows >= kStreamFromRows && cols >= int64_t(WideShape<D>::kCols) * 128;
+}
+// ... and the narrow form wherever the form above would take four columns per workgroup
+__device__ __forceinline__ bool input_fusion_narrow(int64_t cols) { return cols < 8 * 512; }
+
+// acc + c[0] + c[1] + ... + c[n-1], added in that order, for a column c of kTileRows consecutive floats
+// (16-byte aligned, all of them readable): sixteen rows arrive as four 128-bit LDS reads while the previous
+// sixteen are added, so the adder issues 1.25 instructions per row.
+template <int kTileRows>
+__device__ __forceinline__ float add_column_in_row_order(float acc, const float *c, int n) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  f32x4 x[4], y[4];
+  auto read16 = [&](f32x4(&v)[4], int r) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      v[q] = *reinterpret_cast<const f32x4 *>(c + r + 4 * q);
+  };
+  auto add16 = [&](const f32x4(&v)[4]) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      acc = acc + v[q].x;
+      acc = acc + v[q].y;
+      acc = acc + v[q].z;
+      acc = acc + v[q].w;
+    }
+  };
+  int r = 0;
+  read16(x, 0);
+  for (; r + 32 <= n; r += 32) {
+    read16(y, r + 16);
+    add16(x);
+    read16(x, r + 32 < kTileRows ? r + 32 : 0); // past the tile's last row: any readable rows, not added
+    add16(y);
+  }
+  // x holds rows r .. r + 15; fewer than 32 rows are left
+  if (r + 16 <= n) {
+    read16(y, r + 16);
+    add16(x);
+    r += 16;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (r + 4 * q + e < n)
+          acc = acc + y[q][e];
+  } else {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (r + 4 * q + e < n)
+          acc = acc + x[q][e];
+  }
+  return acc;
 }
 
-template <Dt D>
+template <Dt D, typename S>
 __device__ __forceinline__ void input_fusion_stream(const void *__restrict__ a, const void *__restrict__ b,
                                                     void *__restrict__ out, int64_t rows, int64_t cols,
                                                     const LogfEntry *table, float *tile) {
   using E = Elem<D>;
-  using S = StreamShape<D>;
-  constexpr int kCols = S::kCols, kTileRows = S::kTileRows, kPasses = S::kPasses;
+  constexpr int kCols = S::kCols, kTileRows = S::kTileRows, kWorkers = S::kWork, kPer = S::kPer;
+  constexpr int kGroupPasses = S::kGroupPasses;
+  struct Raw { // what one load brings: a 16-byte vector, or one element already widened
+    u32x4 v;
+    float f;
+  };
   const int tid = threadIdx.x;
   const int64_t tiles = (rows + kTileRows - 1) / kTileRows;
+  const int64_t groups = (tiles + S::kGroupTiles - 1) / S::kGroupTiles;
   for (int64_t c0 = int64_t(blockIdx.x) * kCols; c0 < cols; c0 += int64_t(gridDim.x) * kCols) {
-    if (tid < kStreamWorkers) {
-      const int lr = tid >> 3, lc = (tid & 7) * E::kPerVec; // row within an access, first column of the lane's vector
+    if (tid < kWorkers) {
+      const int lr = tid / S::kLanes, lc = (tid % S::kLanes) * kPer; // row within a pass, the lane's first column
       // Rows past the end and, in a partial last block, columns past the end re-read a position inside the
       // matrix instead (their results are never added): the loads are then unconditional, straight-line
-      // code, and the wait for a tile's data leaves the next tile's loads in flight.
-      const int64_t colOff = c0 + lc < cols ? c0 + lc : c0; // cols is a multiple of the vector: all of it or none
-      const char *pa = static_cast<const char *>(a) + colOff * E::kBytes;
-      const char *pb = static_cast<const char *>(b) + colOff * E::kBytes;
-      u32x4 ca[kPasses], cb[kPasses], na[kPasses], nb[kPasses];
-      auto load_tile = [&](int64_t t, u32x4(&va)[kPasses], u32x4(&vb)[kPasses]) {
+      // code, and the wait for a tile's data leaves the next group's loads in flight.
+      const int64_t col = c0 + lc < cols ? c0 + lc : c0; // vectors: cols is a multiple of the vector, all of it or none
+      Raw ca[kGroupPasses], cb[kGroupPasses], na[kGroupPasses], nb[kGroupPasses];
+      auto load_group = [&](int64_t g, Raw(&va)[kGroupPasses], Raw(&vb)[kGroupPasses]) {
 #pragma unroll
-        for (int p = 0; p < kPasses; ++p) {
-          const int64_t r = min(t * kTileRows + p * S::kRowsPerPass + lr, rows - 1);
-          va[p] = load128<true>(reinterpret_cast<const u32x4 *>(pa + r * cols * E::kBytes));
-          vb[p] = load128<true>(reinterpret_cast<const u32x4 *>(pb + r * cols * E::kBytes));
+        for (int p = 0; p < kGroupPasses; ++p) {
+          const int64_t r = min((g * kGroupPasses + p) * S::kRowsPerPass + lr, rows - 1);
+          if constexpr (S::kVec) {
+            va[p].v = load128<true>(reinterpret_cast<const u32x4 *>(static_cast<const char *>(a) + (r * cols + col) * E::kBytes));
+            vb[p].v = load128<true>(reinterpret_cast<const u32x4 *>(static_cast<const char *>(b) + (r * cols + col) * E::kBytes));
+          } else {
+            va[p].f = E::get(a, r * cols + col);
+            vb[p].f = E::get(b, r * cols + col);
+          }
         }
       };
-      load_tile(0, ca, cb);
-      for (int64_t t = 0; t < tiles; ++t) {
-        load_tile(t + 1 < tiles ? t + 1 : t, na, nb); // past the last tile: the last one again, unused
-        float *dst = tile + (t & 1) * kStreamTileElems + lr * kCols + lc;
+      load_group(0, ca, cb);
+      for (int64_t g = 0; g < groups; ++g) {
+        load_group(g + 1 < groups ? g + 1 : g, na, nb); // past the last group: the last one again, unused
 #pragma unroll
-        for (int p = 0; p < kPasses; ++p) {
-          float fa[E::kPerVec], fb[E::kPerVec];
-          E::unpack(ca[p], fa);
-          E::unpack(cb[p], fb);
-          bool ordinary = true;
+        for (int j = 0; j < S::kGroupTiles; ++j) {
+          const int64_t t = g * S::kGroupTiles + j;
+          if (t < tiles) { // uniform
+            float *dst = tile + (t & 1) * S::kTileFloats + lc * S::kColPitch + lr;
 #pragma unroll
-          for (int i = 0; i < E::kPerVec; ++i)
-            ordinary = ordinary && logf_ordinary(fb[i]);
-          if (__builtin_amdgcn_ballot_w64(!ordinary) == 0) { // uniform over the wavefront
+            for (int q = 0; q < S::kTilePasses; ++q) {
+              const int p = j * S::kTilePasses + q;
+              float fa[kPer], fb[kPer];
+              if constexpr (S::kVec) {
+                E::unpack(ca[p].v, fa);
+                E::unpack(cb[p].v, fb);
+              } else {
+                fa[0] = ca[p].f;
+                fb[0] = cb[p].f;
+              }
+              bool ordinary = true;
 #pragma unroll
-            for (int i = 0; i < E::kPerVec; ++i)
-              fa[i] = input_chain<true>(fa[i], fb[i], table);
-          } else {
+              for (int i = 0; i < kPer; ++i)
+                ordinary = ordinary && logf_ordinary(fb[i]);
+              if (__builtin_amdgcn_ballot_w64(!ordinary) == 0) { // uniform over the wavefront
 #pragma unroll
-            for (int i = 0; i < E::kPerVec; ++i)
-              fa[i] = input_chain(fa[i], fb[i], table);
+                for (int i = 0; i < kPer; ++i)
+                  fa[i] = input_chain<true>(fa[i], fb[i], table);
+              } else {
+#pragma unroll
+                for (int i = 0; i < kPer; ++i)
+                  fa[i] = input_chain(fa[i], fb[i], table);
+              }
+#pragma unroll
+              for (int i = 0; i < kPer; ++i)
+                dst[i * S::kColPitch + q * S::kRowsPerPass] = fa[i];
+            }
+            __syncthreads(); // tile t is complete; the adder is done with tile t-1, whose buffer tile t+1 goes into
           }
-          u32x4 *d = reinterpret_cast<u32x4 *>(dst + p * S::kRowsPerPass * kCols);
-#pragma unroll
-          for (int i = 0; i < E::kPerVec / 4; ++i)
-            d[i] = u32x4{f2u(fa[4 * i]), f2u(fa[4 * i + 1]), f2u(fa[4 * i + 2]), f2u(fa[4 * i + 3])};
         }
-        __syncthreads(); // tile t is complete; the adder is done with tile t-1, whose buffer tile t+1 goes into
 #pragma unroll
-        for (int p = 0; p < kPasses; ++p) {
+        for (int p = 0; p < kGroupPasses; ++p) {
           ca[p] = na[p];
           cb[p] = nb[p];
         }
       }
     } else {
-      const int col = tid - kStreamWorkers;
+      const int col = tid - kWorkers;
       const bool active = col < kCols && c0 + col < cols;
       float acc = 0.0f;
       for (int64_t t = 0; t < tiles; ++t) {
         __syncthreads(); // tile t is complete
         const int n = rows - t * kTileRows < kTileRows ? int(rows - t * kTileRows) : kTileRows;
         if (active)
-          acc = add_in_row_order(acc, tile + (t & 1) * kStreamTileElems + col, n, kCols);
+          acc = add_column_in_row_order<kTileRows>(acc, tile + (t & 1) * S::kTileFloats + col * S::kColPitch, n);
       }
       if (active)
         E::put(out, c0 + col, acc);
@@ -390,13 +486,17 @@ template <Dt D>
 __device__ __forceinline__ void input_fusion(const void *__restrict__ a, const void *__restrict__ b,
                                              void *__restrict__ out, int64_t rows, int64_t cols) {
   __shared__ LogfEntry table[16];
-  __shared__ __attribute__((aligned(16))) float tile[2 * kStreamTileElems];
+  __shared__ __attribute__((aligned(16))) float tile[2 * kStreamTileFloats];
   stage_table(table);
-  // The launch says which form: 576 lanes ask for the streaming one, which needs whole aligned vectors.
+  // The launch says which form: 576 or 320 lanes ask for a streaming one, which needs whole aligned vectors.
   const bool vectors = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0 &&
                        cols % Elem<D>::kPerVec == 0;
   if (blockDim.x == kStreamThreads && vectors && input_fusion_streams<D>(rows, cols)) {
-    input_fusion_stream<D>(a, b, out, rows, cols, table, tile);
+    input_fusion_stream<D, WideShape<D>>(a, b, out, rows, cols, table, tile);
+    return;
+  }
+  if (blockDim.x == kNarrowThreads && input_fusion_narrow(cols)) {
+    input_fusion_stream<D, NarrowShape<D>>(a, b, out, rows, cols, table, tile);
     return;
   }
   switch (input_fusion_block_cols(cols)) {

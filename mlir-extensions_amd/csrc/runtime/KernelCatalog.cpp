@@ -255,7 +255,14 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
       grid[0] = ceilDiv(cols, segment_cols);
       break;
     }
-    // otherwise a workgroup per block of 64 .. 4 columns: the widest that leaves 512 workgroups
+    // Fewer than 4096 columns (the reference's 512 x 1024): the same form with 256 workers and the adder
+    // wavefront = 320 lanes per four columns.
+    if (cols < 8 * 512) {
+      block[0] = 320;
+      grid[0] = ceilDiv(cols, 4);
+      break;
+    }
+    // otherwise a workgroup per block of 64 .. 8 columns: the widest that leaves 512 workgroups
     const int64_t block_cols = cols >= 64 * 512 ? 64 : cols >= 32 * 512 ? 32 : cols >= 16 * 512 ? 16 : cols >= 8 * 512 ? 8 : 4;
     grid[0] = ceilDiv(cols, block_cols);
     break;

@@ -488,8 +488,10 @@ def test_loop_fusion_16bit(host, orc, stream, dtype):
 
 # from 2048 x 4096 on the launch asks for the streaming form (576 lanes): whole tiles, ragged rows and a partial
 # last block of columns, and a column count that is not made of whole vectors (the kernel falls back by itself)
-@pytest.mark.parametrize("shape", [(512, 1024), (9, 5), (1000, 300), (3, 2049), (2048, 4096), (2500, 4100),
-                                   (2049, 4098)])
+# below 4096 columns: four columns per workgroup, 64-row tiles, eight tiles' loads together (one group, several
+# groups, a partial last tile, a partial last block of columns)
+@pytest.mark.parametrize("shape", [(512, 1024), (9, 5), (1000, 300), (3, 2049), (1500, 36), (513, 4), (2048, 4096),
+                                   (2500, 4100), (2049, 4098)])
 def test_input_fusion_f32_bit_exact(host, orc, stream, shape):
     """kInputFusion: column sums in row order from +0.0, as the reference adds them."""
     n = int(np.prod(shape))
@@ -501,7 +503,7 @@ def test_input_fusion_f32_bit_exact(host, orc, stream, shape):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("shape", [(512, 1024), (2048, 8192), (2100, 8200)])
+@pytest.mark.parametrize("shape", [(512, 1024), (700, 41), (2048, 8192), (2100, 8200)])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_input_fusion_16bit(host, orc, stream, dtype, shape):
     rows, cols = shape

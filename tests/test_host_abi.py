@@ -112,7 +112,9 @@ def test_launch_shapes(host):
     assert ls("imex_flash_attention_fwd_f16", [16, 4096])[:2] == ((16, 16, 1), (1024, 1, 1))  # 256 queries: 16 wavefronts
     assert ls("imex_flash_attention_fwd_f16", [64, 1024])[:2] == ((4, 64, 1), (1024, 1, 1))
     assert ls("imex_flash_attention_fwd_f16", [3, 256])[0] == (4, 3, 1)
-    assert ls("imex_input_fusion_f32", [512, 1024])[0] == (256, 1, 1)      # 4 columns per workgroup
+    assert ls("imex_input_fusion_f32", [512, 1024])[:2] == ((256, 1, 1), (320, 1, 1))  # 4 columns per workgroup
+    assert ls("imex_input_fusion_bf16", [512, 1024])[:2] == ((256, 1, 1), (320, 1, 1))
+    assert ls("imex_input_fusion_f32", [512, 4096])[:2] == ((512, 1, 1), (256, 1, 1))
     assert ls("imex_input_fusion_f32", [512, 65536])[0] == (1024, 1, 1)    # 64
     # tall and wide: the streaming form, 576 lanes per 128-byte row segment
     assert ls("imex_input_fusion_f32", [8192, 8192])[:2] == ((256, 1, 1), (576, 1, 1))
