@@ -20,9 +20,11 @@
 // Arguments:  loop fusion  (a, b, out, n: i64)              dims = {n}
 //             input fusion (a, b, out, rows: i64, cols: i64) dims = {rows, cols}
 // Launch: block (256,1,1); loop fusion grid ceil(n / 4096) (f32) or ceil(n / 8192)
-// (16-bit), a quarter of that per workgroup below 4 Mi elements; input fusion grid ceil(cols / c), a workgroup per block of c = 64 .. 4 columns
-// (the widest that leaves 512 workgroups), or, from 2048 rows and 128 row segments of 128 bytes on, block
-// (576,1,1) and grid ceil(cols * element bytes / 128): the streaming form.  Workgroups stride, so any grid is correct.
+// (16-bit), a quarter of that per workgroup below 4 Mi elements.  Input fusion, by shape: below 4096 columns
+// block (320,1,1), grid ceil(cols / 4); from 2048 rows and 128 row segments of 128 bytes on block (576,1,1),
+// grid ceil(cols * element bytes / 128); otherwise block (256,1,1), grid ceil(cols / c), a workgroup per
+// block of c = 64 .. 8 columns (the widest that leaves 512 workgroups).  A launch with 256 lanes always gets
+// the last form.  Workgroups stride, so any grid is correct.
 
 #include "device_common.h"
 
