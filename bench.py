@@ -355,6 +355,40 @@ def measure_reference_suite(stream):
     return out
 
 
+def vendor_yardstick():
+    """The vendor library's f16 4096^3 GEMM on the headline's operands (same seeds, same distribution), timed
+    the way the headline is: settle launches, then 1000 launches between two events.  torch.mm dispatches to
+    hipBLASLt / rocBLAS; nothing in the product uses either.  What the part sustains on these operand values
+    under a tuned library is the scale the headline's fraction of the 2.5 PFLOP/s peak has to be read on."""
+    import torch
+    M = N = K = 4096
+    a = torch.from_numpy(gen_uniform(M * K, "f16", 20246, -1.0, 1.0).view(np.float16).reshape(M, K)).cuda()
+    b = torch.from_numpy(gen_uniform(K * N, "f16", 20247, -1.0, 1.0).view(np.float16).reshape(K, N)).cuda()
+    results = {}
+    for label, make in (("f16_out", lambda x, y: torch.mm(x, y)),
+                        ("f32_out", lambda x, y: torch.mm(x, y, out_dtype=torch.float32))):
+        for operands, (x, y) in (("uniform", (a, b)), ("zeros", (torch.zeros_like(a), torch.zeros_like(b)))):
+            try:
+                for _ in range(SETTLE_LAUNCHES):
+                    make(x, y)
+                torch.cuda.synchronize()
+                start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                for _ in range(1000):
+                    make(x, y)
+                stop.record()
+                torch.cuda.synchronize()
+                ms = start.elapsed_time(stop) / 1000
+                results["%s_%s" % (label, operands)] = {"ms_per_launch": round(ms, 5),
+                                                        "tflops": round(2.0 * M * N * K / ms / 1e9, 1),
+                                                        "frac_of_2.5_pflops": round(2.0 * M * N * K / ms / 1e9 / 2500.0, 4)}
+            except (RuntimeError, TypeError) as e:  # e.g. a torch build whose mm takes no out_dtype
+                results["%s_%s" % (label, operands)] = {"error": str(e).splitlines()[0][:200]}
+            log("vendor GEMM %s, %s operands: %s" % (label, operands, results["%s_%s" % (label, operands)]))
+    print(json.dumps({"vendor_gemm_f16_4096": results, "library": "torch.mm (torch %s)" % torch.__version__,
+                      "protocol": "%d settle launches, then 1000 launches between two events" % SETTLE_LAUNCHES}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -364,7 +398,13 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline legs")
     ap.add_argument("--suite", action="store_true",
                     help="also time every shape of the reference's benchmark suite (us per launch, back to back)")
+    ap.add_argument("--vendor-yardstick", action="store_true",
+                    help="time the vendor GEMM library (through torch.mm) on the headline's operands and exit: "
+                         "a yardstick printed as its own JSON line, never part of `value`")
     args = ap.parse_args()
+    if args.vendor_yardstick:
+        vendor_yardstick()
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: every kernel here runs on a single MI355X and this build has no "
               "multi-GPU path (--gpus %d refused)" % args.gpus, file=sys.stderr)
