@@ -385,8 +385,58 @@ def vendor_yardstick():
             except (RuntimeError, TypeError) as e:  # e.g. a torch build whose mm takes no out_dtype
                 results["%s_%s" % (label, operands)] = {"error": str(e).splitlines()[0][:200]}
             log("vendor GEMM %s, %s operands: %s" % (label, operands, results["%s_%s" % (label, operands)]))
-    print(json.dumps({"vendor_gemm_f16_4096": results, "library": "torch.mm (torch %s)" % torch.__version__,
-                      "protocol": "%d settle launches, then 1000 launches between two events" % SETTLE_LAUNCHES}))
+    # The memory-bound configurations through the same library's own kernels, on the rotating protocol (a ring
+    # of separate tensor sets of at least 2 GiB, every result written into a preallocated tensor of its set).
+    def rotating(make_set, op, algorithmic_bytes, set_bytes):
+        sets = [make_set() for _ in range(max(2, -(-(2 << 30) // set_bytes)))]
+        for st in sets:
+            op(*st)
+        torch.cuda.synchronize()
+        passes = max(2, 200 // len(sets))
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(passes):
+            for st in sets:
+                op(*st)
+        stop.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(stop) / (passes * len(sets))
+        return {"ms_per_launch": round(ms, 5), "frac_of_8_TBps": round(algorithmic_bytes / ms / 1e6 / 8000.0, 4)}
+
+    def randn(shape, dtype):
+        return torch.randn(shape, device="cuda", dtype=torch.float32).to(dtype)
+
+    streaming = {}
+    cases = (
+        ("relu_f32_4096x4096", lambda: (randn((4096, 4096), torch.float32), torch.empty((4096, 4096), device="cuda")),
+         lambda x, y: torch.clamp_min(x, 0.0, out=y), 2 * 4096 * 4096 * 4, 2 * 4096 * 4096 * 4),
+        ("softmax_f16_16384x1024",
+         lambda: (randn((16384, 1024), torch.float16), torch.empty((16384, 1024), device="cuda", dtype=torch.float16)),
+         lambda x, y: torch.softmax(x, 1, out=y), 2 * 16384 * 1024 * 2, 2 * 16384 * 1024 * 2),
+        ("rowsum_f32_8192x8192", lambda: (randn((8192, 8192), torch.float32), torch.empty((8192,), device="cuda")),
+         lambda x, y: torch.sum(x, 1, out=y), 8192 * 8192 * 4 + 8192 * 4, 8192 * 8192 * 4),
+        ("transpose_bf16_8192x8192",
+         lambda: (randn((8192, 8192), torch.bfloat16), torch.empty((8192, 8192), device="cuda", dtype=torch.bfloat16)),
+         lambda x, y: y.copy_(x.t()), 2 * 8192 * 8192 * 2, 2 * 8192 * 8192 * 2),
+        ("transpose_f32_4096x4096",
+         lambda: (randn((4096, 4096), torch.float32), torch.empty((4096, 4096), device="cuda")),
+         lambda x, y: y.copy_(x.t()), 2 * 4096 * 4096 * 4, 2 * 4096 * 4096 * 4),
+        ("silu_f32_512x640x20x15",
+         lambda: (randn((98304000,), torch.float32), torch.empty((98304000,), device="cuda")),
+         lambda x, y: torch.ops.aten.silu.out(x, out=y), 2 * 98304000 * 4, 2 * 98304000 * 4),
+    )
+    for name, make_set, op, algorithmic, set_bytes in cases:
+        try:
+            streaming[name] = rotating(make_set, op, algorithmic, set_bytes)
+        except (RuntimeError, TypeError) as e:
+            streaming[name] = {"error": str(e).splitlines()[0][:200]}
+        torch.cuda.empty_cache()
+        log("vendor %s: %s" % (name, streaming[name]))
+    print(json.dumps({"vendor_gemm_f16_4096": results, "vendor_streaming_rotating": streaming,
+                      "library": "torch %s (mm, clamp_min, softmax, sum, copy_ of a transposed view, silu)" % torch.__version__,
+                      "protocol": "GEMM: %d settle launches, then 1000 launches between two events; streaming: a ring of "
+                                  "tensor sets of at least 2 GiB, one settle pass, then about 200 launches between two events"
+                                  % SETTLE_LAUNCHES}))
 
 
 def main():
