@@ -385,6 +385,33 @@ def vendor_yardstick():
             except (RuntimeError, TypeError) as e:  # e.g. a torch build whose mm takes no out_dtype
                 results["%s_%s" % (label, operands)] = {"error": str(e).splitlines()[0][:200]}
             log("vendor GEMM %s, %s operands: %s" % (label, operands, results["%s_%s" % (label, operands)]))
+    # The MLP-shaped configuration: the library's bf16 GEMM alone (bf16 output, no bias, no activation), and with
+    # the bias add and SiLU as the framework's separate kernels after it.
+    Mm, Km, Nm = 4096, 4096, 11008
+    am = torch.from_numpy(gen_normal(Mm * Km, "bf16", 20248, 0.0, 1.0).view(np.int16).reshape(Mm, Km)).cuda().view(torch.bfloat16)
+    bm = torch.from_numpy(gen_normal(Km * Nm, "bf16", 20249, 0.0, 0.02).view(np.int16).reshape(Km, Nm)).cuda().view(torch.bfloat16)
+    biasm = torch.from_numpy(gen_normal(Nm, "f32", 20250, 0.0, 0.1)).cuda()
+    for label, make in (("mlp_bf16_gemm_only", lambda: torch.mm(am, bm)),
+                        ("mlp_bf16_gemm_bias_silu_unfused",
+                         lambda: torch.nn.functional.silu(torch.mm(am, bm).float() + biasm).to(torch.bfloat16))):
+        try:
+            for _ in range(50):
+                make()
+            torch.cuda.synchronize()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(200):
+                make()
+            stop.record()
+            torch.cuda.synchronize()
+            ms = start.elapsed_time(stop) / 200
+            results[label] = {"ms_per_launch": round(ms, 5), "tflops": round(2.0 * Mm * Nm * Km / ms / 1e9, 1),
+                              "frac_of_2.5_pflops": round(2.0 * Mm * Nm * Km / ms / 1e9 / 2500.0, 4)}
+        except (RuntimeError, TypeError) as e:
+            results[label] = {"error": str(e).splitlines()[0][:200]}
+        log("vendor %s: %s" % (label, results[label]))
+    del am, bm
+
     # The memory-bound configurations through the same library's own kernels, on the rotating protocol (a ring
     # of separate tensor sets of at least 2 GiB, every result written into a preallocated tensor of its set).
     def rotating(make_set, op, algorithmic_bytes, set_bytes):
