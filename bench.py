@@ -412,6 +412,27 @@ def vendor_yardstick():
         log("vendor %s: %s" % (label, results[label]))
     del am, bm
 
+    # Flash-attention forward, head dimension 64, f16, no mask: the framework's fused attention.
+    for label, (z, h, n_ctx) in (("attention_f16_2x2x4096x64", (2, 2, 4096)), ("attention_f16_16x4096x64", (1, 16, 4096))):
+        try:
+            q, k, v = (torch.randn((z, h, n_ctx, 64), device="cuda", dtype=torch.float32).to(torch.float16) for _ in range(3))
+            for _ in range(50):
+                torch.nn.functional.scaled_dot_product_attention(q, k, v)
+            torch.cuda.synchronize()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(300):
+                torch.nn.functional.scaled_dot_product_attention(q, k, v)
+            stop.record()
+            torch.cuda.synchronize()
+            ms = start.elapsed_time(stop) / 300
+            flop = 4.0 * z * h * n_ctx * n_ctx * 64
+            results[label] = {"ms_per_launch": round(ms, 5), "tflops": round(flop / ms / 1e9, 1),
+                              "frac_of_2.5_pflops": round(flop / ms / 1e9 / 2500.0, 4)}
+        except (RuntimeError, TypeError) as e:
+            results[label] = {"error": str(e).splitlines()[0][:200]}
+        log("vendor %s: %s" % (label, results[label]))
+
     # The memory-bound configurations through the same library's own kernels, on the rotating protocol (a ring
     # of separate tensor sets of at least 2 GiB, every result written into a preallocated tensor of its set).
     def rotating(make_set, op, algorithmic_bytes, set_bytes):
