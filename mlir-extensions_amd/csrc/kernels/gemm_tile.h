@@ -128,21 +128,36 @@ struct StoreF32 {       // C = acc
     C[m * N + n] = acc; // ordinary store: C stays in the last-level cache for whoever reads it next
   }
 };
+// Epilogues that read C first also offer the two halves separately -- fetch() the old value, put() the new one
+// computed from it -- so that the tiled path can issue a whole batch of reads before the first dependent store
+// (element by element, every read would wait for the store before it: C may alias itself).
 struct AccumulateF32 {  // C = C + acc   (the reference kernel loads C as its initial accumulator)
   static constexpr bool kColumnsInRegisters = false;
+  static constexpr bool kReadsC = true;
   float *C;
+  __device__ __forceinline__ float fetch(int64_t m, int64_t n, int64_t N) const { return C[m * N + n]; }
+  __device__ __forceinline__ void put(int64_t m, int64_t n, int64_t N, float acc, float old) const {
+    C[m * N + n] = old + acc;
+  }
   __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
-    C[m * N + n] = C[m * N + n] + acc;
+    put(m, n, N, acc, fetch(m, n, N));
   }
 };
 struct BiasAccumulateF32 { // C = bias[n] + (C + acc)  (bias.mlir:88-94,112-113)
   static constexpr bool kColumnsInRegisters = false;
+  static constexpr bool kReadsC = true;
   float *C;
   const float *bias;
+  __device__ __forceinline__ float fetch(int64_t m, int64_t n, int64_t N) const { return C[m * N + n]; }
+  __device__ __forceinline__ void put(int64_t m, int64_t n, int64_t N, float acc, float old) const {
+    C[m * N + n] = bias[n] + (old + acc);
+  }
   __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
-    C[m * N + n] = bias[n] + (C[m * N + n] + acc);
+    put(m, n, N, acc, fetch(m, n, N));
   }
 };
+template <typename Epi, typename = void> struct ReadsC { static constexpr bool value = false; };
+template <typename Epi> struct ReadsC<Epi, decltype(void(Epi::kReadsC))> { static constexpr bool value = Epi::kReadsC; };
 // v / (1 + exp(-v)) with the hardware's exponential and reciprocal estimates (about an ulp each):
 // the result is rounded to bf16, 2^-9 relative, straight afterwards.
 __device__ __forceinline__ float silu_fast(float v) { return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
@@ -539,6 +554,35 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
           asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1"
                        : "+v"(acc[i][j][r]), "+v"(acc[i][j + 1][r])); // -> rows r, r+8 | rows r+4, r+12
         }
+    if constexpr (ReadsC<Epi>::value) {
+      if (interior) {
+        // the old values of row block i + 1 are requested before row block i is combined and stored
+        float old[2][FJ * 4];
+        auto fetch_block = [&](int i, float(&into)[FJ * 4]) {
+#pragma unroll
+          for (int j = 0; j < FJ; j += 2)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              into[j * 4 + r] = epi.fetch(mBase + i * 16 + r, nBase + j * 16, N);
+              into[j * 4 + 4 + r] = epi.fetch(mBase + i * 16 + r + 4, nBase + j * 16, N);
+            }
+        };
+        fetch_block(0, old[0]);
+#pragma unroll
+        for (int i = 0; i < FI; ++i) {
+          if (i + 1 < FI)
+            fetch_block(i + 1, old[(i + 1) & 1]);
+#pragma unroll
+          for (int j = 0; j < FJ; j += 2)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              epi.put(mBase + i * 16 + r, nBase + j * 16, N, acc[i][j][r], old[i & 1][j * 4 + r]);
+              epi.put(mBase + i * 16 + r + 4, nBase + j * 16, N, acc[i][j + 1][r], old[i & 1][j * 4 + 4 + r]);
+            }
+        }
+        return;
+      }
+    }
     if (interior) {
 #pragma unroll
       for (int i = 0; i < FI; ++i)
