@@ -416,7 +416,8 @@ __device__ __forceinline__ void input_fusion_stream(const void *__restrict__ a, 
           }
         }
       };
-      load_group(0, ca, cb);
+      if (groups > 0) // (no rows: nothing to read, the sums are +0.0)
+        load_group(0, ca, cb);
       for (int64_t g = 0; g < groups; ++g) {
         load_group(g + 1 < groups ? g + 1 : g, na, nb); // past the last group: the last one again, unused
 #pragma unroll

@@ -471,6 +471,8 @@ def test_fused_chains_empty_and_single(host, orc, stream):
     assert host.loop_fusion(stream, empty, empty).shape == (0,)
     one = host.loop_fusion(stream, np.float32([2.5]), np.float32([-1.5]))
     assert np.array_equal(one, orc.loop_fusion_f32(np.float32([2.5]), np.float32([-1.5])))
+    no_rows = host.input_fusion(stream, np.zeros((0, 12), np.float32), np.zeros((0, 12), np.float32))
+    assert np.array_equal(no_rows.view(np.uint32), np.zeros(12, np.uint32))  # a sum over nothing: +0.0
     col = host.input_fusion(stream, np.float32([[1.0], [-2.0], [3.0]]), np.float32([[0.5], [2.0], [8.0]]))
     assert np.array_equal(col, orc.input_fusion_f32(np.float32([[1.0], [-2.0], [3.0]]), np.float32([[0.5], [2.0], [8.0]])))
 
