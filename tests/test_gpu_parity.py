@@ -516,6 +516,29 @@ def test_input_fusion_16bit(host, orc, stream, dtype, shape):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("shape,block", [((600, 520), 320), ((2048, 4160), 576), ((2048, 4160), 256), ((600, 520), 256)])
+def test_input_fusion_any_grid(host, orc, stream, shape, block):
+    """Workgroups stride over the blocks of columns in every form of the kernel (the narrow and the wide
+    streaming form, and the 256-lane form a launch with 256 lanes always gets): a grid of a few
+    workgroups gives the same bits as the catalogue's."""
+    import ctypes as C
+    rows, cols = shape
+    a = orc.fill_uniform(rows * cols, "f32", 51, -5.0, 5.0).reshape(shape)
+    b = orc.fill_uniform(rows * cols, "f32", 52, 0.01, 40.0).reshape(shape)
+    want = orc.input_fusion_f32(a, b)
+    d_a, d_b, d_out = stream.to_device(a), stream.to_device(b), stream.alloc(cols * 4)
+    fn = stream.kernel("imex_input_fusion_f32")
+    descs, keep = host._pack_params([d_a, d_b, d_out, rows, cols])
+    for grid in (1, 7):
+        stream.memset(d_out, 0x7fc00000, cols, 32)
+        stream.rt.gpuLaunchKernel(stream.handle, fn, grid, 1, 1, block, 1, 1, 0, C.cast(descs, C.c_void_p), None)
+        stream.wait()
+        got = stream.from_device(d_out, (cols,), np.float32)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (shape, block, grid)
+    for p in (d_a, d_b, d_out):
+        stream.free(p)
+
+
 # ============================ flash attention ===============================
 def attention_close(got_bits, ref_bits, orc):
     """The reference checks its kernel with allclose (atol 1e-4, rtol 1e-3) on a constant
