@@ -3,7 +3,7 @@
 // blocking and the reference kernels it stands for are described in gemm_tile.h.
 //
 // Launch: block (512,1,1); grid (tiles,1,1) with tiles = ceil(M/256)*ceil(N/256) on
-// the MFMA path, else (ceil(M*N/512),1,1); workgroups stride, so any grid is correct.  The fixed-shape
+// the MFMA path, else (ceil(M/128)*ceil(N/128),1,1); workgroups stride, so any grid is correct.  The fixed-shape
 // 4096^3 entry points take the reference's own launch: blocks (16,16,1), threads (512,1,1).
 
 #include "gemm_tile.h"

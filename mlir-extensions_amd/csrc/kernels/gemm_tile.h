@@ -47,12 +47,12 @@
 // in place of the missing ones and store only what is inside C.  What the MFMA path
 // does need is 16-byte aligned rows in memory (K % 8 == 0; N % 8 == 0
 // where B is [K,N], M % 8 == 0 where A is [K,M]; a K that does not fill the last 32-wide step is
-// padded with zeros on the way into LDS); other shapes take the
-// one-thread-per-output path of the same kernels, which adds in ascending k like the
+// padded with zeros on the way into LDS); other shapes take the vector-ALU path of the
+// same kernels (128 x 128 tiles, gemm_blocked), which adds in ascending k like the
 // reference's CPU loop (lib/ExecutionEngine/ImexRunnerUtils.cpp:308-317).
 //
 // Launch: block (512,1,1); grid (tiles,1,1) with tiles = ceil(M/256)*ceil(N/256) on
-// the MFMA path, else (ceil(M*N/512),1,1); workgroups stride, so any grid is correct.  The fixed-shape 4096^3 entry
+// the MFMA path, else (ceil(M/128)*ceil(N/128),1,1); workgroups stride, so any grid is correct.  The fixed-shape 4096^3 entry
 // points take the reference's own launch: blocks (16,16,1), threads (512,1,1).
 
 #ifndef IMEX_HIP_GEMM_TILE_H
@@ -203,25 +203,71 @@ struct StoreF16 {       // C(f16) = acc   (WG/gemm_4kx4kx4k_f16_f16_f16.mlir)
   }
 };
 
-// ---- one-thread-per-output path ---------------------------------------------------
-// kAT: A is stored [K,M] (A[k*M+m]) instead of [M,K]; kBT: B is stored [N,K]
-// (B[n*K+k]) instead of [K,N].
+// ---- any-shape path: 128 x 128 tiles on the vector ALUs -----------------------------------
+// For operands the MFMA path cannot take (rows that are not 16-byte aligned in memory).  Every output is
+// the reference's CPU loop (lib/ExecutionEngine/ImexRunnerUtils.cpp:308-317): acc = 0, then for ascending
+// k a rounded multiply and a rounded add (this file is built with contraction off), so the result is the
+// oracle's bit for bit; the tiling only shares the operand loads.  512 lanes hold 8 x 4 outputs each; A
+// and B go through LDS sixteen k at a time, widened to f32, zero beyond M, N and K (a zero product leaves
+// the sum as it is: the sum starts at +0.0 and never becomes -0.0).
+// kAT: A is stored [K,M] (A[k*M+m]) instead of [M,K]; kBT: B is stored [N,K] (B[n*K+k]) instead of [K,N].
 template <typename T, bool kAT, bool kBT, typename Epi>
-__device__ __forceinline__ void gemm_scalar(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
-                                            Epi epi) {
-  // grid-stride, so that any launch shape covers every output
-  const int64_t block = int64_t(blockIdx.y) * gridDim.x + blockIdx.x;
-  const int64_t stride = int64_t(gridDim.x) * gridDim.y * kThreads;
-  for (int64_t idx = block * kThreads + threadIdx.x; idx < M * N; idx += stride) {
-    const int64_t m = idx / N, n = idx % N;
-    float acc = 0.0f;
-    for (int64_t k = 0; k < K; ++k) {
-      const float a = T::widen(kAT ? A[k * M + m] : A[m * K + k]);
-      const float b = T::widen(kBT ? B[n * K + k] : B[k * N + n]);
-      const float p = a * b;
-      acc = acc + p; // rounded multiply, rounded add (file is built with contraction off)
+__device__ __forceinline__ void gemm_blocked(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
+                                             Epi epi, char *ldsBytes) {
+  constexpr int TM = 128, TN = 128, TK = 16, kPitch = TM + 4; // the pad keeps a k-fastest fill off one bank
+  float(*As)[kPitch] = reinterpret_cast<float(*)[kPitch]>(ldsBytes);
+  float(*Bs)[kPitch] = reinterpret_cast<float(*)[kPitch]>(ldsBytes + TK * kPitch * sizeof(float));
+  const int tid = threadIdx.x, tx = tid & 31, ty = tid >> 5; // columns 4 tx .., rows 8 ty ..
+  const int64_t tilesN = (N + TN - 1) / TN, tiles = ((M + TM - 1) / TM) * tilesN;
+  const int64_t workgroups = int64_t(gridDim.x) * gridDim.y;
+  for (int64_t id = int64_t(blockIdx.y) * gridDim.x + blockIdx.x; id < tiles; id += workgroups) {
+    const int64_t m0 = (id / tilesN) * TM, n0 = (id % tilesN) * TN;
+    float acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = 0.0f;
+    for (int64_t k0 = 0; k0 < K; k0 += TK) {
+      __syncthreads(); // the previous k block has been read
+#pragma unroll
+      for (int u = 0; u < TM * TK / kThreads; ++u) {
+        const int e = u * kThreads + tid;
+        // the index that is contiguous in memory varies fastest over the lanes
+        const int am = kAT ? e % TM : e / TK, ak = kAT ? e / TM : e % TK;
+        const int64_t m = m0 + am, k = k0 + ak;
+        As[ak][am] = m < M && k < K ? T::widen(kAT ? A[k * M + m] : A[m * K + k]) : 0.0f;
+        const int bn = kBT ? e / TK : e % TN, bk = kBT ? e % TK : e / TN;
+        const int64_t n = n0 + bn, kb = k0 + bk;
+        Bs[bk][bn] = n < N && kb < K ? T::widen(kBT ? B[n * K + kb] : B[kb * N + n]) : 0.0f;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < TK; ++k) {
+        float a[8], b[4];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          a[i] = As[k][ty * 8 + i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          b[j] = Bs[k][tx * 4 + j];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float p = a[i] * b[j];
+            acc[i][j] = acc[i][j] + p; // rounded multiply, rounded add
+          }
+      }
     }
-    epi(m, n, N, acc);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t m = m0 + ty * 8 + i, n = n0 + tx * 4 + j;
+        if (m < M && n < N)
+          epi(m, n, N, acc[i][j]);
+      }
   }
 }
 
@@ -343,7 +389,7 @@ template <typename T, bool kStrided, int kFrags, bool kTail> struct Operand {
   }
 };
 
-// kAT / kBT as in gemm_scalar.  A is KContig unless transposed; B is KContig only
+// kAT / kBT as in gemm_blocked.  A is KContig unless transposed; B is KContig only
 // when transposed.
 // One 256 x 256 tile of C: tile number `id` of a tilesM x tilesN grid.
 template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0, bool kTail = false>
@@ -645,7 +691,7 @@ __device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B,
   else if (tileable)
     gemm_tiled<T, kAT, kBT, Epi, kProbe, true>(A, B, M, N, K, epi, lds);
   else
-    gemm_scalar<T, kAT, kBT, Epi>(A, B, M, N, K, epi);
+    gemm_blocked<T, kAT, kBT, Epi>(A, B, M, N, K, epi, lds);
 }
 
 } // namespace imexhip_gemm

@@ -272,7 +272,7 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
   case Shape::GemmTB: {
     // 512 lanes: eight wavefronts per 256 x 256 tile of C, edge tiles included.  The MFMA path
     // needs 16-byte aligned rows in memory, i.e. K % 8 == 0, N % 8 == 0 where B is [K,N] and
-    // M % 8 == 0 where A is [K,M]; everything else is one lane per output.
+    // M % 8 == 0 where A is [K,M]; everything else runs 128 x 128 tiles on the vector ALUs.
     const int64_t M = dims[0], N = dims[1], K = dims[2];
     const bool rowsB = e->shape == Shape::GemmTB || N % 8 == 0;
     const bool rowsA = e->shape != Shape::GemmTA || M % 8 == 0;
@@ -282,7 +282,7 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     const bool fitsB = e->shape == Shape::GemmTB ? K < maxRow : K * N * 2 < twoGiB;
     const bool tileable = M > 0 && N > 0 && K > 0 && K % 8 == 0 && rowsA && rowsB && fitsA && fitsB;
     block[0] = 512;
-    grid[0] = tileable ? ceilDiv(M, 256) * ceilDiv(N, 256) : ceilDiv(M * N, 512);
+    grid[0] = tileable ? ceilDiv(M, 256) * ceilDiv(N, 256) : ceilDiv(M, 128) * ceilDiv(N, 128);
     break;
   }
   case Shape::GemmFixed4k: // the reference's own launch: blocks (16,16,1), threads (512,1,1)

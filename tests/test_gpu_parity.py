@@ -710,13 +710,30 @@ def test_gemm_golden_3x3(host, orc, stream):
     assert np.all(orc.half_to_float(out) == g["expected_fill"])
 
 
-@pytest.mark.parametrize("M,N,K", [(5, 7, 9), (100, 36, 130), (256, 256, 20), (256, 256, 44), (255, 252, 64), (17, 300, 64)])
-def test_gemm_untileable_shapes_bit_exact(host, orc, stream, M, N, K):
-    """K not a multiple of 8 or N not a multiple of 8: the one-lane-per-output path, which
-    accumulates in the oracle's order."""
-    a = orc.fill_uniform(M * K, "f16", 1, -1, 1).reshape(M, K)
-    b = orc.fill_uniform(K * N, "f16", 2, -1, 1).reshape(K, N)
-    assert np.array_equal(host.gemm(stream, a, b, ab_dtype="f16"), orc.gemm(a, b, "f16"))
+@pytest.mark.parametrize("M,N,K", [(5, 7, 9), (100, 36, 130), (256, 256, 20), (256, 256, 44), (255, 252, 64), (17, 300, 64),
+                                   (300, 260, 50), (129, 129, 17)])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_untileable_shapes_bit_exact(host, orc, stream, M, N, K, dtype):
+    """K not a multiple of 8 or N not a multiple of 8: the vector-ALU path (128 x 128 tiles, sixteen k at a
+    time), which accumulates every output in the oracle's order."""
+    a = orc.fill_uniform(M * K, dtype, 1, -1, 1).reshape(M, K)
+    b = orc.fill_uniform(K * N, dtype, 2, -1, 1).reshape(K, N)
+    assert np.array_equal(host.gemm(stream, a, b, ab_dtype=dtype), orc.gemm(a, b, dtype))
+
+
+def test_gemm_untileable_special_values(host, orc, stream):
+    """The vector-ALU path pads its tiles with zeros beyond M, N and K; infinities, NaNs and negative zeros
+    in the operands must come out as in the sequential loop, which never sees the padding."""
+    M, N, K = 70, 37, 21
+    a = orc.fill_uniform(M * K, "f16", 3, -1, 1).reshape(M, K)
+    b = orc.fill_uniform(K * N, "f16", 4, -1, 1).reshape(K, N)
+    a[3, 5], a[9, 20], a[60, 0], a[69, 20] = 0x7c00, 0xfc00, 0x7e00, 0x7c00      # +inf, -inf, NaN, +inf
+    b[20, 36], b[0, 0] = 0x7c00, 0xfc00
+    a[11, :] = 0x8000                                                         # a row of -0.0
+    got, want = host.gemm(stream, a, b, ab_dtype="f16"), orc.gemm(a, b, "f16")
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(got.view(np.uint32)[ok], want.view(np.uint32)[ok])
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
@@ -845,7 +862,7 @@ def test_gemm_ragged_tiles_transposed_operands(host, orc, stream, which, M, N, K
 
 def test_gemm_launch_shape_slack(host, orc, stream):
     """A grid with more or fewer workgroups than tiles (MFMA path: the workgroups stride
-    over the tiles) or fewer threads than outputs (one-thread-per-output path) still
+    over the tiles) or fewer workgroups than tiles (vector-ALU path) still
     computes every element once."""
     import ctypes as C
     for (M, N, K, grid) in [(256, 256, 64, 9), (100, 36, 130, 2), (1024, 768, 96, 5), (1000, 520, 64, 1)]:
@@ -902,8 +919,8 @@ def test_gemm_transposed_operands(host, orc, stream, which):
     def stored(a, b):
         return (np.ascontiguousarray(a.T), b) if which == "ta" else (a, np.ascontiguousarray(b.T))
 
-    # one-thread-per-output path: bit-exact against the sequential oracle
-    for (M, N, K) in [(5, 7, 9), (100, 36, 130)]:
+    # vector-ALU path: bit-exact against the sequential oracle
+    for (M, N, K) in [(5, 7, 9), (100, 36, 130), (300, 260, 50)]:
         a = orc.fill_uniform(M * K, "f16", 31, -1, 1).reshape(M, K)
         b = orc.fill_uniform(K * N, "f16", 32, -1, 1).reshape(K, N)
         sa, sb = stored(a, b)

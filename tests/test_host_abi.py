@@ -93,13 +93,13 @@ def test_launch_shapes(host):
     assert ls("imex_gemm_f16_f16_f32", [255, 256, 64])[0] == (1, 1, 1)
     assert ls("imex_gemm_f16_f16_f32", [257, 520, 64])[0] == (6, 1, 1)
     assert ls("imex_gemm_f16_f16_f32", [256, 256, 48])[0] == (1, 1, 1)     # K % 32 != 0 but K % 8 == 0: still tiled
-    assert ls("imex_gemm_f16_f16_f32", [256, 256, 44])[0] == (128, 1, 1)   # K % 8 != 0: one lane per output
-    assert ls("imex_gemm_f16_f16_f32", [256, 252, 64])[0] == (126, 1, 1)   # N % 8 != 0
+    assert ls("imex_gemm_f16_f16_f32", [256, 256, 44])[0] == (4, 1, 1)     # K % 8 != 0: 128 x 128 vector-ALU tiles
+    assert ls("imex_gemm_f16_f16_f32", [256, 252, 64])[0] == (4, 1, 1)     # N % 8 != 0
     assert ls("imex_gemm_f16_f16_f32_tb", [256, 252, 64])[0] == (1, 1, 1)  # B stored [N,K]: any N
-    assert ls("imex_gemm_f16_f16_f32_ta", [252, 256, 64])[0] == (126, 1, 1)  # A stored [K,M]: M % 8 != 0
+    assert ls("imex_gemm_f16_f16_f32_ta", [252, 256, 64])[0] == (4, 1, 1)    # A stored [K,M]: M % 8 != 0
     assert ls("imex_gemm_f16_f16_f32_ta", [248, 256, 64])[0] == (1, 1, 1)
-    # a strided operand of 2 GiB or more cannot be addressed with 32-bit offsets: one lane per output
-    assert ls("imex_gemm_f16_f16_f32", [256, 32768, 32768])[0] == (256 * 32768 // 512, 1, 1)
+    # a strided operand of 2 GiB or more cannot be addressed with 32-bit offsets: the vector-ALU tiles
+    assert ls("imex_gemm_f16_f16_f32", [256, 32768, 32768])[0] == (2 * 256, 1, 1)
     assert ls("imex_gemm_f16_f16_f32", [256, 32768, 32736])[0] == (128, 1, 1)
     assert ls("imex_gemm_f16_f16_f32_tb", [256, 32768, 32768])[0] == (128, 1, 1)
     assert ls("imex_gemm_4kx4kx4k_f16_f16_f32", []) == ((16, 16, 1), (512, 1, 1), 0)
@@ -342,7 +342,7 @@ def test_launch_shapes_cover_the_problem(host):
             (gx, gy, gz), block, _ = ls(name, [M, N, K])
             assert block == (512, 1, 1) and gy == gz == 1
             tileable = K % 8 == 0 and (name.endswith("_tb") or N % 8 == 0) and (not name.endswith("_ta") or M % 8 == 0)
-            assert gx == -(-M // 256) * -(-N // 256) if tileable else gx * 512 >= M * N
+            assert gx == (-(-M // 256) * -(-N // 256) if tileable else -(-M // 128) * -(-N // 128))
 
     eltwise()
     rowwise()
