@@ -25,3 +25,14 @@ def test_generators_match_the_oracle(orc, dtype):
     got, want = bench.gen_bits(n, dtype, 20244), orc.fill_bits(n, dtype, 20244)
     assert np.array_equal(got.view(np.uint32 if dtype == "f32" else np.uint16),
                           want.view(np.uint32 if dtype == "f32" else np.uint16))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """Every figure of this build is one GPU's: `bench.py --gpus N` with N > 1 says so and exits before it
+    touches a device."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(REPO, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE,
+                       stderr=subprocess.PIPE, text=True, timeout=120)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
