@@ -56,20 +56,34 @@ template <bool kStream> __device__ __forceinline__ void store128(u32x4 v, u32x4 
     *p = v;
 }
 
-// Butterfly reductions across the 64 lanes of a wavefront.  The xor shuffles
-// lower to DPP row operations for distances < 16 and to lane permutes above.
+// Reductions across the 64 lanes of a wavefront, every lane active, on the VALU's own
+// cross-lane paths (DPP): four steps inside each row of 16 lanes (quad swaps, half-row and row
+// mirrors: afterwards every lane holds its row's result), two row broadcasts (rows 1 and 3 take
+// lane 15 of the row before, rows 2 and 3 take lane 31; the row mask leaves the other rows as they
+// are), and lane 63 read out as a wavefront-uniform value.  Seven instructions and no LDS round
+// trip; the xor-shuffle form costs six dependent ds_bpermute.  Written as instructions: from the
+// builtins the compiler made a copy, a canonicalising maximum and the maximum itself out of every
+// step.  A DPP operand must not be read for two wait states after a VALU wrote it, hence the
+// s_nop before each step (the compiler cannot see hazards inside an asm block); the trailing one
+// covers whatever reads the result next.
+#define IMEX_DPP_REDUCE(op)                                                                                   \
+  "s_nop 1\n\t" op " %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"                            \
+  "s_nop 1\n\t" op " %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"                            \
+  "s_nop 1\n\t" op " %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"                                \
+  "s_nop 1\n\t" op " %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"                                     \
+  "s_nop 1\n\t" op " %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"                                   \
+  "s_nop 1\n\t" op " %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"                                   \
+  "s_nop 1"
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1)
-    v += __shfl_xor(v, off, kWave);
-  return v;
+  asm volatile(IMEX_DPP_REDUCE("v_add_f32_dpp") : "+v"(v));
+  return u2f(__builtin_amdgcn_readlane(f2u(v), 63));
 }
+// NaN operands are passed over (v_max_f32 returns the other operand), like fmaxf.
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1)
-    v = fmaxf(v, __shfl_xor(v, off, kWave));
-  return v;
+  asm volatile(IMEX_DPP_REDUCE("v_max_f32_dpp") : "+v"(v));
+  return u2f(__builtin_amdgcn_readlane(f2u(v), 63));
 }
+#undef IMEX_DPP_REDUCE
 
 // Element traits for kernels that exist in f32, f16 and bf16 forms: scalar get / put through
 // f32, and a 16-byte vector (u32x4) unpacked to / packed from kPerVec f32 values.  16-bit values

@@ -183,6 +183,162 @@ __device__ __forceinline__ void softmax_rows_in_regs(const void *in, void *out, 
   }
 }
 
+// ---- f16 rows in registers: the benchmark's path, written for the instruction count ----------
+// At [16384,1024] every SIMD has 16384 elements to get through while 64 MiB stream past: the
+// vector instructions per element, not the memory system, decide the run time.  Per element:
+//   maximum       v_pk_max_f16 on the packed input words (exact in f16)                   1/2
+//   exponent      one v_fma_mix_f32 straight from the f16 half: x*log2(e) - m*log2(e)      1
+//   exponential   v_exp_f32 (quarter rate)                                                1
+//   row sum       v_add_f32                                                               1
+//   normalise     v_fma_mixlo/hi_f16: e * (1/sum), rounded to f16 into its half           1
+// and no conversion instruction on either side.  m*log2(e) is rounded once per row; the error
+// of that rounding multiplies every exponential of the row by the same factor and leaves the
+// quotients alone.  f16 only: |m| <= 65504 keeps m*log2(e) finite (a bf16 or f32 maximum near
+// 3e38 would not), and a row of nothing but -inf still comes out NaN (fma(-inf, c, +inf)), as
+// the reference's 0/0 does.  Outputs are >= +0, so folding the final multiplication into the
+// rounding instruction cannot lose a sign.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+constexpr float kLog2e = 1.44269504088896340736f;
+
+// The instruction itself: the builtin maximum puts a canonicalising v_pk_max_f16 x, x in front of
+// every operand that comes from memory.  A NaN is passed over or (a signalling one) returned quiet;
+// the row comes out all-NaN either way, through the sum.
+__device__ __forceinline__ f16x2 pk_max_f16(f16x2 a, f16x2 b) {
+  f16x2 d;
+  asm("v_pk_max_f16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+
+// One row of up to 1024 columns held by a wavefront as two 16-byte vectors per lane.
+struct F16Row {
+  u32x4 raw[kRegChunks];
+
+  // kFull: the row is exactly 1024 columns.  Otherwise lanes whose vector lies past the end of the
+  // row load the row's first vector instead (no lane is switched off, so the compiler can count the
+  // loads in flight) and are given -inf afterwards, which the maximum and the sum pass over.
+  template <bool kFull> __device__ __forceinline__ void load(const char *rowBase, int lane, int vecsPerRow) {
+#pragma unroll
+    for (int c = 0; c < kRegChunks; ++c) {
+      const int v = c * kWave + lane;
+      const int vc = kFull || v < vecsPerRow ? v : 0;
+      raw[c] = load128<true>(reinterpret_cast<const u32x4 *>(rowBase) + vc);
+    }
+  }
+
+  // kSite: a different number at every call site.  It goes into the code as a comment, which keeps
+  // the compiler from merging the ends of two call sites into one block: the merged block waited for
+  // every memory operation of every path into it, stores of the row before included.
+  template <bool kFull, int kSite>
+  __device__ __forceinline__ void softmax_and_store(char *rowBase, int lane, int vecsPerRow) {
+    constexpr uint32_t kMinusInfPair = 0xfc00fc00u;
+    f16x2 h[kRegChunks * 4];
+#pragma unroll
+    for (int c = 0; c < kRegChunks; ++c) {
+      const bool live = kFull || c * kWave + lane < vecsPerRow;
+      // (through named words: a bit cast applied directly to a vector component reads component 0)
+      const uint32_t w0 = live ? raw[c].x : kMinusInfPair, w1 = live ? raw[c].y : kMinusInfPair,
+                     w2 = live ? raw[c].z : kMinusInfPair, w3 = live ? raw[c].w : kMinusInfPair;
+      h[4 * c + 0] = __builtin_bit_cast(f16x2, w0);
+      h[4 * c + 1] = __builtin_bit_cast(f16x2, w1);
+      h[4 * c + 2] = __builtin_bit_cast(f16x2, w2);
+      h[4 * c + 3] = __builtin_bit_cast(f16x2, w3);
+    }
+    f16x2 m2 = pk_max_f16(pk_max_f16(pk_max_f16(h[0], h[1]), pk_max_f16(h[2], h[3])),
+                          pk_max_f16(pk_max_f16(h[4], h[5]), pk_max_f16(h[6], h[7])));
+    static_assert(kRegChunks == 2, "the maximum above is written out for eight words");
+    // lanes past the end of a short row hold -inf; the reference's maximum starts at kMaxInit
+    const float m = fmaxf(wave_max(fmaxf(static_cast<float>(m2.x), static_cast<float>(m2.y))), kMaxInit);
+    const float negMl2 = -(m * kLog2e);
+    float e[kRegChunks * 8];
+#pragma unroll
+    for (int i = 0; i < kRegChunks * 4; ++i) {
+      e[2 * i] = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(h[i].x), kLog2e, negMl2));
+      e[2 * i + 1] = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(h[i].y), kLog2e, negMl2));
+    }
+    float s0 = e[0], s1 = e[1];
+#pragma unroll
+    for (int i = 1; i < kRegChunks * 4; ++i) {
+      s0 += e[2 * i];
+      s1 += e[2 * i + 1];
+    }
+    const float s = wave_sum(s0 + s1);
+    // one reciprocal per row (the hardware's estimate and a Newton step: within an ulp of 1 / s),
+    // then multiplies; s = 0, inf or NaN all give a NaN row, like the reference's division
+    float inv = __builtin_amdgcn_rcpf(s);
+    inv = __builtin_fmaf(__builtin_fmaf(-s, inv, 1.0f), inv, inv);
+#pragma unroll
+    for (int c = 0; c < kRegChunks; ++c) {
+      const int v = c * kWave + lane;
+      uint32_t w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const f16x2 p = {static_cast<_Float16>(__builtin_fmaf(e[8 * c + 2 * i], inv, 0.0f)),
+                         static_cast<_Float16>(__builtin_fmaf(e[8 * c + 2 * i + 1], inv, 0.0f))};
+        w[i] = __builtin_bit_cast(uint32_t, p);
+      }
+      asm volatile("; softmax row, call site %0, vector %1" ::"n"(kSite), "n"(c));
+      if (kFull || v < vecsPerRow)
+        store128<true>(u32x4{w[0], w[1], w[2], w[3]}, reinterpret_cast<u32x4 *>(rowBase) + v);
+    }
+    asm volatile("; softmax row done, call site %0" ::"n"(kSite));
+  }
+};
+
+// The walk: wavefront w of W takes rows w, w + W, w + 2W, ... and always has its next row's loads
+// in flight while it works on the current one -- reads, vector work and writes of different rows
+// overlap inside a wavefront as well as between wavefronts.  The loads are unconditional
+// straight-line code in a branch of their own ("there is a next row" is uniform), so the wait in
+// front of a row's arithmetic is for that row's two loads only and leaves the next row's in flight.
+// Any grid is correct; the catalogue's grid gives every wavefront slot of the chip one wavefront.
+template <bool kFull>
+__device__ __forceinline__ void softmax_f16_rows_in_regs(const void *in, void *out, int64_t rows, int64_t cols) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t stride = int64_t(gridDim.x) * kWaves;
+  const int vecsPerRow = static_cast<int>(cols / 8);
+  const int64_t rowBytes = cols * 2;
+  const char *src = static_cast<const char *>(in);
+  char *dst = static_cast<char *>(out);
+  // the wavefront's number as a scalar, so that row addresses are formed on the scalar unit
+  int64_t row = int64_t(blockIdx.x) * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  if (row >= rows || vecsPerRow == 0)
+    return;
+  F16Row a, b;
+  a.load<kFull>(src + row * rowBytes, lane, vecsPerRow);
+  if (row + stride >= rows) {
+    a.softmax_and_store<kFull, 1>(dst + row * rowBytes, lane, vecsPerRow);
+    return;
+  }
+  // The first row is taken outside the loop so that the loop is entered, the first time and every
+  // later time, with the same memory operations in flight (a row's loads, then the row before's two
+  // stores): the wait counts inside are then exact and never wait for a store.
+  b.load<kFull>(src + (row + stride) * rowBytes, lane, vecsPerRow);
+  __builtin_amdgcn_sched_barrier(0); // the loads stay in front of the wait for the current row
+  a.softmax_and_store<kFull, 2>(dst + row * rowBytes, lane, vecsPerRow);
+  row += stride;
+  for (;;) {
+    // b holds `row`
+    if (row + stride < rows) {
+      a.load<kFull>(src + (row + stride) * rowBytes, lane, vecsPerRow);
+      __builtin_amdgcn_sched_barrier(0);
+      b.softmax_and_store<kFull, 3>(dst + row * rowBytes, lane, vecsPerRow);
+    } else {
+      b.softmax_and_store<kFull, 4>(dst + row * rowBytes, lane, vecsPerRow);
+      return;
+    }
+    row += stride;
+    // a holds `row`
+    if (row + stride < rows) {
+      b.load<kFull>(src + (row + stride) * rowBytes, lane, vecsPerRow);
+      __builtin_amdgcn_sched_barrier(0);
+      a.softmax_and_store<kFull, 5>(dst + row * rowBytes, lane, vecsPerRow);
+    } else {
+      a.softmax_and_store<kFull, 6>(dst + row * rowBytes, lane, vecsPerRow);
+      return;
+    }
+    row += stride;
+  }
+}
+
 // ---- workgroup reductions -------------------------------------------------------------
 __device__ __forceinline__ float block_reduce(float v, bool isMax, float *scratch) {
   v = isMax ? wave_max(v) : wave_sum(v);
@@ -344,7 +500,12 @@ __device__ __forceinline__ void softmax_kernel(const void *in, void *out, int64_
                        (cols % E::kPerVec) == 0;
   if (aligned && cols <= int64_t(kRegChunks) * kWave * E::kPerVec) {
     // non-temporal accesses: measured faster hot and cold
-    if (rows >= kTwoRowsFrom)
+    if constexpr (D == Dt::F16) {
+      if (cols == int64_t(kRegChunks) * kWave * 8)
+        softmax_f16_rows_in_regs<true>(in, out, rows, cols);
+      else
+        softmax_f16_rows_in_regs<false>(in, out, rows, cols);
+    } else if (rows >= kTwoRowsFrom)
       softmax_rows_in_regs<D, true, 2>(in, out, rows, cols);
     else
       softmax_rows_in_regs<D, true, 1>(in, out, rows, cols);

@@ -168,12 +168,19 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     break;
   case Shape::SoftmaxRows32:
   case Shape::SoftmaxRows16: {
-    // Rows of up to 128 x 16 B stay in registers, one per wavefront (four per
-    // workgroup; two per wavefront from 16384 rows on); longer rows take a workgroup each.  The kernel strides over
-    // the rows, so any grid is correct; this one covers them in a single pass.
+    // Rows of up to 128 x 16 B stay in registers, one per wavefront (four per workgroup); longer rows take
+    // a workgroup each.  The kernels stride over the rows, so any grid is correct.  f32 and bf16 register
+    // rows: one pass (two rows per wavefront from 16384 rows on).  f16 register rows: a wavefront walks
+    // its rows with the next row's loads in flight, and 2048 workgroups give every wavefront slot of the
+    // chip (256 CUs x 4 SIMDs x 8) one wavefront.
     const int64_t regCols = e->shape == Shape::SoftmaxRows16 ? 1024 : 512;
-    grid[0] = dims[1] <= regCols ? ceilDiv(dims[0], dims[0] >= 16384 ? 8 : 4)
-                                 : static_cast<size_t>(dims[0] < 1048560 ? dims[0] : 1048560);
+    const bool f16 = std::strcmp(e->name, "imex_softmax_f16") == 0;
+    if (dims[1] > regCols)
+      grid[0] = static_cast<size_t>(dims[0] < 1048560 ? dims[0] : 1048560);
+    else if (f16)
+      grid[0] = std::min<size_t>(ceilDiv(dims[0], 4), 2048);
+    else
+      grid[0] = ceilDiv(dims[0], dims[0] >= 16384 ? 8 : 4);
     if (dims[1] == 0)
       grid[0] = 0;
     break;

@@ -232,6 +232,29 @@ def test_softmax_nan_and_infinite_rows(host, orc, stream, dtype, cols):
     assert np.all(np.abs(got[ok] - ref[ok]) <= 1e-3 * np.abs(ref[ok]) + (2.0 ** -24 if dtype == "f16" else 0.0))
 
 
+@pytest.mark.parametrize("rows,cols", [(1000, 1024), (1000, 1016), (37, 1024), (4097, 1024), (5, 8)])
+def test_softmax_f16_rows_in_registers_any_grid(host, orc, stream, rows, cols):
+    """The f16 register path walks its rows with the next row's loads in flight: a wavefront that takes one
+    row, two, three (odd and even trip counts of the two-row loop) or a few hundred gives the same bits as
+    the catalogue's grid, for whole 1024-column rows and for rows that leave lanes without a vector."""
+    say("softmax f16 walk %dx%d" % (rows, cols))
+    x = orc.fill_normal(rows * cols, "f16", 7 * rows + cols, 0.0, 2.0).reshape(rows, cols)
+    x[rows // 2, cols // 2] = 0x7E00  # a NaN row in the middle of a walk
+    ref = orc.softmax_16(x, "f16")
+    want = host.softmax(stream, x, "f16")
+    nan = np.isnan(orc.half_to_float(ref))
+    assert np.array_equal(np.isnan(orc.half_to_float(want)), nan) and nan[rows // 2].all() and nan.sum() == cols
+    ok = ~nan
+    assert close_16(orc, want[ok], ref[ok], "f16")
+    for grid in (1, 2, -(-rows // 12), -(-rows // 8), -(-rows // 4) + 3):
+        d_in, d_out = stream.to_device(x), stream.alloc(rows * cols * 2)
+        stream.launch("imex_softmax_f16", [rows, cols], [d_in, d_out, rows, cols], grid=(grid, 1, 1))
+        stream.wait()
+        got = stream.from_device(d_out, (rows, cols), np.uint16)
+        stream.free(d_in), stream.free(d_out)
+        assert np.array_equal(got[ok], want[ok]) and np.isnan(orc.half_to_float(got[~ok])).all(), grid
+
+
 # =============================== Reductions ================================
 def test_rowsum_golden_and_exact(host, orc, stream):
     g = GOLD["sum_f32_10x20"]

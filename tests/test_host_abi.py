@@ -65,8 +65,11 @@ def test_launch_shapes(host):
     assert ls("imex_exp_f32", [256 * 256]) == ((64, 1, 1), (256, 1, 1), 0)  # one vector per lane below 4 Mi elements
     assert ls("imex_relu_f32", [0])[0][0] == 0  # nothing to launch
     assert ls("imex_relu_bf16", [8193])[0] == (2, 1, 1)
-    assert ls("imex_softmax_f16", [16384, 1024])[0] == (2048, 1, 1)  # two rows per wavefront from 16384 rows on
-    assert ls("imex_softmax_f16", [16383, 1024])[0] == (4096, 1, 1)
+    assert ls("imex_softmax_f16", [16384, 1024])[0] == (2048, 1, 1)  # a wavefront per slot of the chip; they walk the rows
+    assert ls("imex_softmax_f16", [16383, 1024])[0] == (2048, 1, 1)
+    assert ls("imex_softmax_f16", [1000, 512])[0] == (250, 1, 1)
+    assert ls("imex_softmax_bf16", [16384, 1024])[0] == (2048, 1, 1)  # two rows per wavefront from 16384 rows on
+    assert ls("imex_softmax_bf16", [16383, 1024])[0] == (4096, 1, 1)
     assert ls("imex_softmax_f32", [16, 2000])[0] == (16, 1, 1)
     assert ls("imex_rowsum_f32", [8192, 8192])[0] == (8192, 1, 1)
     assert ls("imex_rowsum_f32", [8, 256])[0] == (2, 1, 1)
@@ -329,6 +332,8 @@ def test_launch_shapes_cover_the_problem(host):
         (gx, _, _), _, _ = ls("imex_input_fusion_f32", [rows, cols])
         assert gx * 64 >= cols
         (gx, _, _), _, _ = ls("imex_softmax_f16", [rows, cols])
+        assert gx >= 1 and (gx == min(-(-rows // 4), 2048) if cols <= 1024 else gx >= min(rows, 1048560))
+        (gx, _, _), _, _ = ls("imex_softmax_bf16", [rows, cols])
         assert gx >= 1 and (gx * (8 if rows >= 16384 else 4) >= rows if cols <= 1024 else gx >= min(rows, 1048560))
 
     @settings(max_examples=300, deadline=None)
