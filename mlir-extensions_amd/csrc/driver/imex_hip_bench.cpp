@@ -68,7 +68,8 @@ struct Workload {
   double work;                  // algorithmic bytes or flops per launch
   bool mfma;                    // roofline: MFMA (TFLOP/s) or HBM (GB/s)
   bool probe = false;           // a measurement kernel: loaded from imex_probe.hsaco beside this program
-  int probeGrid = 0;            // its grid (workgroups of 512 lanes); 0: one lane per dims[0]
+  int probeGrid = 0;            // its grid (workgroups of probeBlock lanes); 0: one lane per dims[0]
+  int probeBlock = 512;
 };
 
 std::vector<Workload> workloads() {
@@ -180,6 +181,12 @@ std::vector<Workload> workloads() {
       {"gemm_f16_4096_probe_multiply_only", "imex_gemm_probe_multiply_only", {},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_f16_4096_probe_store_nontemporal", "imex_gemm_probe_store_nontemporal", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_f16_4096_probe_store_lines", "imex_gemm_probe_store_lines", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
       {"gemm_f16_4096_probe_copies_only", "imex_gemm_probe_copies_only", {},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
@@ -189,8 +196,92 @@ std::vector<Workload> workloads() {
       {"gemm_f16_4096_probe_copies_only_b", "imex_gemm_probe_copies_only_b", {},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_f16_4096_probe_narrow_a", "imex_gemm_probe_narrow_a", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_f16_4096_probe_narrow_a_copies_only", "imex_gemm_probe_narrow_a_copies_only", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_f16_4096_probe_narrow_a_copies_only_a", "imex_gemm_probe_narrow_a_copies_only_a", {},
+       {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
+       {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      // the 16-bit transpose's traffic without the transposition: 256 x 256 tiles copied to their own / to the
+      // transposed tile position, at the benchmark's 16 KiB row pitch and at 32 KiB; and the transpose itself at 32 KiB
+      {"tile_copy_b16_8192x8192_own", "imex_probe_tile_copy_b16", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8, 0}, 0,
+       2.0 * K8 * K8 * 2, false, true, 32 * 32, 256},
+      {"tile_copy_b16_8192x8192_transposed", "imex_probe_tile_copy_b16", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8, 1}, 0,
+       2.0 * K8 * K8 * 2, false, true, 32 * 32, 256},
+      {"tile_copy_b16_16384x16384_own", "imex_probe_tile_copy_b16", {2 * K8, 2 * K8},
+       {{Elem::BF16, {2 * K8, 2 * K8}, true, -1, 1}, {Elem::BF16, {2 * K8, 2 * K8}, false, 0, 0}}, {2 * K8, 2 * K8, 0}, 0,
+       2.0 * 4 * K8 * K8 * 2, false, true, 64 * 64, 256},
+      {"tile_copy_b16_16384x16384_transposed", "imex_probe_tile_copy_b16", {2 * K8, 2 * K8},
+       {{Elem::BF16, {2 * K8, 2 * K8}, true, -1, 1}, {Elem::BF16, {2 * K8, 2 * K8}, false, 0, 0}}, {2 * K8, 2 * K8, 1}, 0,
+       2.0 * 4 * K8 * K8 * 2, false, true, 64 * 64, 256},
+      // the traffic of a tile-wise 16-bit transpose for other tile shapes (R x C: 2 C-byte read, 2 R-byte write segments)
+      {"tile_traffic_b16_8192x8192_256x256", "imex_probe_tile_traffic_b16_256x256", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, 0,
+       2.0 * K8 * K8 * 2, false, true, int(K8 / 256 * K8 / 256), 256},
+      {"tile_traffic_b16_8192x8192_128x128", "imex_probe_tile_traffic_b16_128x128", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, 0,
+       2.0 * K8 * K8 * 2, false, true, int(K8 / 128 * K8 / 128), 256},
+      {"tile_traffic_b16_8192x8192_512x128", "imex_probe_tile_traffic_b16_512x128", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, 0,
+       2.0 * K8 * K8 * 2, false, true, int(K8 / 512 * K8 / 128), 256},
+      {"tile_traffic_b16_8192x8192_128x512", "imex_probe_tile_traffic_b16_128x512", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, 0,
+       2.0 * K8 * K8 * 2, false, true, int(K8 / 128 * K8 / 512), 256},
+      {"tile_traffic_b16_8192x8192_512x256", "imex_probe_tile_traffic_b16_512x256", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, 0,
+       2.0 * K8 * K8 * 2, false, true, int(K8 / 512 * K8 / 256), 512},
+      {"tile_traffic_b16_8192x8192_256x512", "imex_probe_tile_traffic_b16_256x512", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, 0,
+       2.0 * K8 * K8 * 2, false, true, int(K8 / 256 * K8 / 512), 512},
+      {"tile_traffic_b16_8192x8192_1024x128", "imex_probe_tile_traffic_b16_1024x128", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, 0,
+       2.0 * K8 * K8 * 2, false, true, int(K8 / 1024 * K8 / 128), 512},
+      {"tile_traffic_b16_8192x8192_512x512", "imex_probe_tile_traffic_b16_512x512", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8}, 0,
+       2.0 * K8 * K8 * 2, false, true, int(K8 / 512 * K8 / 512), 1024},
+      // reads alone and writes alone at the two pitches (half the bytes of a copy each), and the copy with a pass's rows spread out
+      {"tile_read_b16_8192x16384", "imex_probe_tile_copy_b16", {K8, 2 * K8},
+       {{Elem::BF16, {K8, 2 * K8}, true, -1, 1}, {Elem::BF16, {K8, 2 * K8}, false, 0, 0}}, {K8, 2 * K8, 2}, 0,
+       2.0 * K8 * K8 * 2, false, true, 32 * 64, 256},
+      {"tile_read_b16_16384x8192", "imex_probe_tile_copy_b16", {2 * K8, K8},
+       {{Elem::BF16, {2 * K8, K8}, true, -1, 1}, {Elem::BF16, {2 * K8, K8}, false, 0, 0}}, {2 * K8, K8, 2}, 0,
+       2.0 * K8 * K8 * 2, false, true, 64 * 32, 256},
+      {"tile_write_b16_8192x16384", "imex_probe_tile_copy_b16", {K8, 2 * K8},
+       {{Elem::BF16, {K8, 2 * K8}, true, -1, 1}, {Elem::BF16, {K8, 2 * K8}, false, 0, 0}}, {K8, 2 * K8, 3}, 0,
+       2.0 * K8 * K8 * 2, false, true, 32 * 64, 256},
+      {"tile_write_b16_16384x8192", "imex_probe_tile_copy_b16", {2 * K8, K8},
+       {{Elem::BF16, {2 * K8, K8}, true, -1, 1}, {Elem::BF16, {2 * K8, K8}, false, 0, 0}}, {2 * K8, K8, 3}, 0,
+       2.0 * K8 * K8 * 2, false, true, 64 * 32, 256},
+      {"tile_copy_b16_16384x8192_own_rows_apart", "imex_probe_tile_copy_b16", {2 * K8, K8},
+       {{Elem::BF16, {2 * K8, K8}, true, -1, 1}, {Elem::BF16, {2 * K8, K8}, false, 0, 0}}, {2 * K8, K8, 4}, 0,
+       2.0 * 2 * K8 * K8 * 2, false, true, 64 * 32, 256},
+      {"tile_copy_b16_8192x8192_transposed_rows_apart", "imex_probe_tile_copy_b16", {K8, K8},
+       {{Elem::BF16, {K8, K8}, true, -1, 1}, {Elem::BF16, {K8, K8}, false, 0, 0}}, {K8, K8, 5}, 0,
+       2.0 * K8 * K8 * 2, false, true, 32 * 32, 256},
+      // equal bytes at the two pitches: 8192 rows of 32 KiB against 16384 rows of 16 KiB
+      {"tile_copy_b16_8192x16384_own", "imex_probe_tile_copy_b16", {K8, 2 * K8},
+       {{Elem::BF16, {K8, 2 * K8}, true, -1, 1}, {Elem::BF16, {K8, 2 * K8}, false, 0, 0}}, {K8, 2 * K8, 0}, 0,
+       2.0 * 2 * K8 * K8 * 2, false, true, 32 * 64, 256},
+      {"tile_copy_b16_16384x8192_own", "imex_probe_tile_copy_b16", {2 * K8, K8},
+       {{Elem::BF16, {2 * K8, K8}, true, -1, 1}, {Elem::BF16, {2 * K8, K8}, false, 0, 0}}, {2 * K8, K8, 0}, 0,
+       2.0 * 2 * K8 * K8 * 2, false, true, 64 * 32, 256},
+      {"transpose_bf16_16384x16384", "imex_transpose2d_b16", {2 * K8, 2 * K8},
+       {{Elem::BF16, {2 * K8, 2 * K8}, 1, -1, 1}, {Elem::BF16, {2 * K8, 2 * K8}, false, 0, 0}}, {2 * K8, 2 * K8}, 0,
+       2.0 * 4 * K8 * K8 * 2, false},
       {"mfma_lds_ceiling_f16_every_exponent", "imex_mfma_lds_ceiling_f16", {256 * 512},
        {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 2}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
+      // the same loop with the operands held in registers (no LDS reads inside it)
+      {"mfma_reg_ceiling_f16_uniform", "imex_mfma_lds_ceiling_f16", {256 * 512},
+       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 4}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
+      {"mfma_reg_ceiling_f16_zeros", "imex_mfma_lds_ceiling_f16", {256 * 512},
+       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 5}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
+      {"mfma_reg_ceiling_f16_every_exponent", "imex_mfma_lds_ceiling_f16", {256 * 512},
+       {{Elem::F32, {256 * 512}, false, 0, 0}}, {256 * 512, 2048, 6}, 0, 256.0 * 8 * 2048 * 32 * 16384, true, true},
   };
 }
 
@@ -247,12 +338,13 @@ int runWorkload(const Workload &w, const Options &opt) {
     }
   }
 
-  size_t grid[3] = {1, 1, 1}, block[3] = {512, 1, 1}, smem = 0;
+  size_t grid[3] = {1, 1, 1}, block[3] = {static_cast<size_t>(w.probeBlock), 1, 1}, smem = 0;
   size_t blobSize = 0;
   const void *blob = nullptr;
   static std::vector<char> probeBlob; // kept for the life of the process: the runtime caches modules by address
   if (w.probe) {
-    grid[0] = w.probeGrid ? static_cast<size_t>(w.probeGrid) : static_cast<size_t>((w.dims[0] + 511) / 512);
+    grid[0] = w.probeGrid ? static_cast<size_t>(w.probeGrid)
+                          : static_cast<size_t>((w.dims[0] + w.probeBlock - 1) / w.probeBlock);
     if (probeBlob.empty()) {
       const std::string path = programDir() + "/imex_probe.hsaco";
       FILE *f = fopen(path.c_str(), "rb");

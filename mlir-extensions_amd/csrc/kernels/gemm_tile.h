@@ -83,9 +83,12 @@ constexpr int WM = BM / kWavesM, WN = BN / kWavesN; // wavefront tile
 constexpr int FI = WM / 16, FJ = WN / 16;           // MFMA 16x16 tiles per wavefront: 8 x 4
 constexpr int kStages = 4;                          // LDS ring: 4 x 32 KiB of the 160 KiB
 constexpr int kImageBytes = 256 * RK * 2;           // one operand's 256 x 32 slab: 16 KiB
-constexpr int kRStage = 2 * kImageBytes;            // A image + B image
 constexpr int kDmaPerWave = kImageBytes / 1024 / kWaves; // 1 KiB global->LDS copies per wavefront, operand and step
 constexpr int kDist = kStages - 1;                  // tiles in flight ahead of the one being multiplied
+constexpr int kRingBytes = kStages * kImageBytes;   // one operand's ring of four slabs: 64 KiB; B's ring first, then A's
+constexpr int kWideStages = 3;                      // A as 64-k-wide slabs (2 x 16 KiB each): a ring of three
+constexpr int kWideBytes = 2 * kImageBytes;
+constexpr int kLdsBytes = kRingBytes + kWideStages * kWideBytes; // 160 KiB: all of a CU's LDS
 constexpr int kGroupM = 4;                          // tile rows per L2-sharing group
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -155,6 +158,24 @@ struct BiasAccumulateF32 { // C = bias[n] + (C + acc)  (bias.mlir:88-94,112-113)
   __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
     put(m, n, N, acc, fetch(m, n, N));
   }
+};
+// f32 results stored 16 bytes per lane from the transposed accumulator (row lane % 16, four consecutive
+// columns): before the stores the upper half-rows (lanes 8-15 of every 16) of column block j trade places
+// with the lower half-rows of block j + 1, after which a lane of block j's registers holds row lane % 8 of
+// block j + (lane % 16) / 8 -- a store instruction then covers eight rows by 128 bytes, whole lines, with a
+// quarter of the store instructions of the element-per-lane form.
+struct StoreF32Lines {
+  static constexpr bool kColumnsInRegisters = true;
+  static constexpr bool kHalfRowExchange = true;
+  float *C;
+  __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const { C[m * N + n] = acc; }
+  __device__ __forceinline__ void vec4(int64_t m, int64_t n, int64_t N, f32x4 acc) const {
+    *reinterpret_cast<f32x4 *>(C + m * N + n) = acc;
+  }
+};
+template <typename Epi, typename = void> struct ExchangesHalfRows { static constexpr bool value = false; };
+template <typename Epi> struct ExchangesHalfRows<Epi, decltype(void(Epi::kHalfRowExchange))> {
+  static constexpr bool value = Epi::kHalfRowExchange;
 };
 template <typename Epi, typename = void> struct ReadsC { static constexpr bool value = false; };
 template <typename Epi> struct ReadsC<Epi, decltype(void(Epi::kReadsC))> { static constexpr bool value = Epi::kReadsC; };
@@ -389,13 +410,56 @@ template <typename T, bool kStrided, int kFrags, bool kTail> struct Operand {
   }
 };
 
+// A k-contiguous operand ([M,K] A) as 64-k-wide slabs: a row of the slab is 128 bytes, one whole L2 line
+// and ONE request to the L2 (the 32-k slab's 64-byte rows go out as twice as many half-line requests --
+// measured: A-only copies 33 us against 26 us for B's 512-byte rows, same bytes).  A slab serves two
+// K-steps and is copied over two steps -- the first 16 of a wavefront's 32 rows at the even step, the
+// rest at the odd one, so every step issues two A and two B copies per wavefront like the 32-k form --
+// into a ring of three.  LDS image [256 rows][64 k]; 16-byte group c of row r at c ^ ((r >> 1) & 7), which
+// keeps the fragment reads (row lane % 16, group 4 p + lane / 16 in the step of parity p) off each
+// other's banks for the lanes the LDS serves together.  One 1 KiB copy = 8 rows.
+template <typename T, int kFrags> struct OperandWide {
+  static constexpr int kCopies = kWideBytes / 1024 / kWaves; // 4
+  __amdgpu_buffer_rsrc_t rsrc;
+  int voff[kCopies];
+  int dstWave;
+  int rd; // parity 0; parity 1 is 64 bytes (four groups) further, i.e. rd ^ 64
+
+  __device__ __forceinline__ void setup(const uint16_t *ptr, int64_t ld, int64_t first, int w0, int64_t extent,
+                                        int wave, int lane) {
+    const int64_t rows = extent / ld - first;
+    const int last = rows < 256 ? int(rows) - 1 : 255;
+    rsrc = make_rsrc(ptr + first * ld, int64_t(last + 1) * ld * 2);
+#pragma unroll
+    for (int q = 0; q < kCopies; ++q) {
+      const int row = wave * (256 / kWaves) + q * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+      voff[q] = int((int64_t(min(row, last)) * ld + chunk * 8) * 2);
+    }
+    dstWave = wave * (256 / kWaves) * (2 * RK * 2);
+    const int fragRow = lane & 15, kGroup = lane >> 4;
+    rd = (w0 + fragRow) * (2 * RK * 2) + ((kGroup ^ ((fragRow >> 1) & 7)) << 4);
+  }
+  // one half (the first or the last 16 of the wavefront's 32 rows) of the wavefront's copies of slab kt2
+  // (K-steps 2 kt2 and 2 kt2 + 1)
+  __device__ __forceinline__ void dma(LdsChar *lds, int image, int kt2, int half) const {
+#pragma unroll
+    for (int q = half * (kCopies / 2); q < (half + 1) * (kCopies / 2); ++q)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + image + dstWave + q * 1024, 16, voff[q], kt2 * (2 * RK * 2), 0, 0);
+  }
+  __device__ __forceinline__ typename T::Frag read(const char *lds, int image, int f, int parity) const {
+    return *reinterpret_cast<const typename T::Frag *>(lds + image + (rd ^ (parity * 64)) + f * 16 * (2 * RK * 2));
+  }
+};
+
 // kAT / kBT as in gemm_blocked.  A is KContig unless transposed; B is KContig only
-// when transposed.
+// when transposed.  kWideA: A's slabs are 64 k wide (A [M,K] and K a multiple of 64 only).
 // One 256 x 256 tile of C: tile number `id` of a tilesM x tilesN grid.
-template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0, bool kTail = false>
+template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0, bool kTail = false, bool kWideA = false>
 __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, int64_t M,
                                           int64_t N, int64_t K, Epi epi, char *lds, int tilesM, int tilesN, int id) {
   static_assert(FI == 8 && FJ == 4 && kWaves == 8, "written for 8 wavefronts of 8 x 4 MFMA tiles");
+  static_assert(!kWideA || (!kAT && !kTail), "wide A slabs: A is [M,K] and K a multiple of 64");
   LdsChar *lds_base = (LdsChar *)lds;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -419,16 +483,28 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   const int lastTile = kTiles - 1;
   const int kRem = int(K - int64_t(lastTile) * RK); // k in the last step: 32, or 8 / 16 / 24 with kTail
   Operand<T, kAT, FI, kTail> opA;
+  OperandWide<T, FI> opAW;
   Operand<T, !kBT, FJ, kTail> opB;
-  opA.setup(A, kAT ? M : K, m0, wm * WM, M * K, waveU, lane, kRem);
+  if constexpr (kWideA)
+    opAW.setup(A, K, m0, wm * WM, M * K, waveU, lane);
+  else
+    opA.setup(A, kAT ? M : K, m0, wm * WM, M * K, waveU, lane, kRem);
   opB.setup(B, kBT ? K : N, n0, wn * WN, K * N, waveU, lane, kRem);
-  constexpr int kImgA = 0, kImgB = kImageBytes;
-  auto dma_tile = [&](int kt, int stageOff) { // stageOff: byte offset of the ring stage, wave-uniform
-    const bool partial = kTail && kt == lastTile;
-    if constexpr (!(kProbe & kProbeNoCopyA))
-      opA.dma(lds_base, stageOff + kImgA, kt, partial);
+  // LDS: B's ring of four 16 KiB slabs at 0, then A's -- four 16 KiB slabs, or three 64-k-wide ones of 32 KiB.
+  // Offsets below are wave-uniform byte offsets of a slab.
+  constexpr int kRingA = kRingBytes;
+  const int lastWide = kTiles / 2 - 1; // (kWideA: kTiles is even)
+  auto dma_a = [&](int kt, int off, int half = 0) { // narrow: K-step kt; wide: one half of 64-k slab kt
+    if constexpr (!(kProbe & kProbeNoCopyA)) {
+      if constexpr (kWideA)
+        opAW.dma(lds_base, off, kt, half);
+      else
+        opA.dma(lds_base, off, kt, kTail && kt == lastTile);
+    }
+  };
+  auto dma_b = [&](int kt, int off) {
     if constexpr (!(kProbe & kProbeNoCopyB))
-      opB.dma(lds_base, stageOff + kImgB, kt, partial);
+      opB.dma(lds_base, off, kt, kTail && kt == lastTile);
   };
 
   // acc[i][j] is the 16 x 16 block at rows 16 i, columns 16 j of the wavefront's tile, held
@@ -447,17 +523,20 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   // (half 1), each by all four B fragments.  af[h] holds half h's A fragments; bf[p] the B
   // fragments of a step of parity p.
   typename T::Frag af[2][FI / 2], bf[2][FJ];
-  auto read_a = [&](int stageOff, int h, int ii) {
+  // off: the slab's byte offset; parity: which half of a wide slab (the K-step's parity)
+  auto read_a = [&](int off, int h, int ii, int parity) {
     if constexpr (kProbe & kProbeCopiesOnly)
       asm volatile("" : "+v"(af[h][ii]));
+    else if constexpr (kWideA)
+      af[h][ii] = opAW.read(lds, off, h * (FI / 2) + ii, parity);
     else
-      af[h][ii] = opA.read(lds, stageOff + kImgA, h * (FI / 2) + ii);
+      af[h][ii] = opA.read(lds, off, h * (FI / 2) + ii);
   };
-  auto read_b = [&](int stageOff, int p, int j) {
+  auto read_b = [&](int off, int p, int j) {
     if constexpr (kProbe & kProbeCopiesOnly)
       asm volatile("" : "+v"(bf[p][j]));
     else
-      bf[p][j] = opB.read(lds, stageOff + kImgB, j);
+      bf[p][j] = opB.read(lds, off, j);
   };
   auto mm = [&](int h, int p, int ii, int j) {
     if constexpr (kProbe & kProbeCopiesOnly)
@@ -471,74 +550,123 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   // A fragments (the fences keep the compiler from regrouping them).  The MFMAs go column
   // block by column block, up and down the row blocks in turn, so that one operand at most
   // changes from one MFMA to the next (fewer operand bits switching: about 1 % on random data).
-  auto half0 = [&](int p, int curOff) {
+  auto half0 = [&](int p, int aCur) {
 #pragma unroll
     for (int j = 0; j < FJ; ++j) {
 #pragma unroll
       for (int s = 0; s < FI / 2; ++s) {
         mm(0, p, (j & 1) ? FI / 2 - 1 - s : s, j);
-        if (s == 0) read_a(curOff, 1, j);
+        if (s == 0) read_a(aCur, 1, j, p);
         IMEX_FENCE();
       }
     }
   };
   // half 1: 16 MFMAs, and between them the reads of the NEXT step's upper A fragments and
   // of its B fragments (into the other parity's registers)
-  auto half1 = [&](int p, int nxtOff) {
+  auto half1 = [&](int p, int aNxt, int bNxt) {
 #pragma unroll
     for (int j = 0; j < FJ; ++j) {
 #pragma unroll
       for (int s = 0; s < FI / 2; ++s) {
         mm(1, p, (j & 1) ? FI / 2 - 1 - s : s, j);
-        if (s == 0) read_a(nxtOff, 0, j);
-        if (s == 2) read_b(nxtOff, p ^ 1, j);
+        if (s == 0) read_a(aNxt, 0, j, p ^ 1);
+        if (s == 2) read_b(bNxt, p ^ 1, j);
         IMEX_FENCE();
       }
     }
   };
 
-  // prologue: tiles 0 .. kDist-1 in flight, tile 0 landed, its first fragments in registers
+  // prologue: tiles 0 .. kDist-1 in flight, tile 0 landed, its first fragments in registers.
+  // Wide A: slabs 0 and 1 (K-steps 0-3) and B's tiles 0-2, issued in the order A0 B0 | A1 (first half) B1 |
+  // A1 (second half) B2 -- the loop's own pattern of two A and two B copies per step -- so that the
+  // same count of copies may stay in flight here and at every step's wait: two steps' worth, eight per wavefront.
+  constexpr int kInFlight = (kDist - 1) * 2 * kDmaPerWave;
+  static_assert(!kWideA || OperandWide<T, FI>::kCopies / 2 == kDmaPerWave, "a wide slab's half is one step's A copies");
   if constexpr (kProbe & kProbeNoLoopCopies) { // every stage filled once, with real operand values
 #pragma unroll
-    for (int t = 0; t < kStages; ++t)
-      dma_tile(min(t, lastTile), t * kRStage);
+    for (int t = 0; t < kStages; ++t) {
+      dma_b(min(t, lastTile), t * kImageBytes);
+      if constexpr (!kWideA)
+        dma_a(min(t, lastTile), kRingA + t * kImageBytes);
+    }
+    if constexpr (kWideA)
+#pragma unroll
+      for (int d = 0; d < kWideStages; ++d) {
+        dma_a(min(d, lastWide), kRingA + d * kWideBytes, 0);
+        dma_a(min(d, lastWide), kRingA + d * kWideBytes, 1);
+      }
     wait_vmcnt<0>();
+  } else if constexpr (kWideA) {
+    dma_a(0, kRingA, 0);
+    dma_a(0, kRingA, 1);
+    dma_b(0, 0);
+    dma_a(min(1, lastWide), kRingA + kWideBytes, 0);
+    dma_b(min(1, lastTile), kImageBytes);
+    dma_a(min(1, lastWide), kRingA + kWideBytes, 1);
+    dma_b(min(2, lastTile), 2 * kImageBytes);
+    if constexpr (kProbe & (kProbeNoCopyA | kProbeNoCopyB))
+      wait_vmcnt<(kDist - 1) * kDmaPerWave>();
+    else
+      wait_vmcnt<kInFlight>();
   } else {
 #pragma unroll
-    for (int t = 0; t < kDist; ++t)
-      dma_tile(min(t, lastTile), t * kRStage);
-    wait_vmcnt<(kDist - 1) * 2 * kDmaPerWave>();
+    for (int t = 0; t < kDist; ++t) {
+      dma_a(min(t, lastTile), kRingA + t * kImageBytes);
+      dma_b(min(t, lastTile), t * kImageBytes);
+    }
+    wait_vmcnt<kInFlight>();
   }
   __builtin_amdgcn_s_barrier();
   IMEX_FENCE();
 #pragma unroll
-  for (int ii = 0; ii < FI / 2; ++ii) read_a(0, 0, ii);
+  for (int ii = 0; ii < FI / 2; ++ii) read_a(kRingA, 0, ii, 0);
 #pragma unroll
   for (int j = 0; j < FJ; ++j) read_b(0, 0, j);
   IMEX_FENCE();
 
-  int curOff = 0;               // stage of tile t
-  int nxtOff = kRStage;         // stage of tile t+1
-  int dmaOff = kDist * kRStage; // stage tile t+kDist goes to (= stage of tile t-1)
+  // slab offsets: B's of tile t, t+1 and the one tile t+kDist goes to (= tile t-1's); A's likewise, or,
+  // wide: the slab of K-steps t and t+1 (t even), the next one, and the one the copies of steps t and
+  // t+1 go to (the slab two ahead = the one that K-steps t-2 and t-1 were read from)
+  int bCur = 0, bNxt = kImageBytes, bDma = kDist * kImageBytes;
+  int aCur = kRingA, aNxt = kRingA + (kWideA ? kWideBytes : kImageBytes);
+  int aDma = kRingA + (kWideA ? 2 * kWideBytes : kDist * kImageBytes);
+  auto next_b = [](int off) { return off + kImageBytes == kRingBytes ? 0 : off + kImageBytes; };
+  auto next_a = [](int off) {
+    constexpr int kSlab = kWideA ? kWideBytes : kImageBytes, kEnd = kRingA + (kWideA ? kWideStages * kWideBytes : kRingBytes);
+    return off + kSlab == kEnd ? kRingA : off + kSlab;
+  };
   auto step = [&](int p, int t) {
-    // The stage of tile t-1 is free: every wavefront passed the previous step's
-    // barrier after its last reads of it.  Past the end of K the copies re-fetch the
-    // last tile into a stage nobody reads, so every step is the same code.
-    if constexpr (!(kProbe & kProbeNoLoopCopies))
-      dma_tile(min(t + kDist, lastTile), dmaOff);
+    // The slabs of tile t-1 are free: every wavefront passed the previous step's
+    // barrier after its last reads of them.  Past the end of K the copies re-fetch the
+    // last tile into a slab nobody reads, so every step is the same code.
+    if constexpr (!(kProbe & kProbeNoLoopCopies)) {
+      if constexpr (kWideA) {
+        dma_a(min(t / 2 + 2, lastWide), aDma, p);
+      } else {
+        dma_a(min(t + kDist, lastTile), aDma);
+      }
+      dma_b(min(t + kDist, lastTile), bDma);
+    }
     IMEX_FENCE();
-    half0(p, curOff);                               // rows 0-63 of tile t; reads its rows 64-127
+    half0(p, aCur);                                 // rows 0-63 of tile t; reads its rows 64-127
     if constexpr (kProbe & (kProbeNoCopyA | kProbeNoCopyB))
       wait_vmcnt<(kDist - 1) * kDmaPerWave>();      // (probe with one operand's copies only)
     else
-      wait_vmcnt<(kDist - 1) * 2 * kDmaPerWave>();  // tile t+1 has landed (this wavefront's part) ...
+      wait_vmcnt<kInFlight>();                      // tile t+1 has landed (this wavefront's part) ...
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();                   // ... and everyone else's; all reads of tile t are done
     IMEX_FENCE();
-    half1(p, nxtOff);                               // rows 64-127 of tile t; reads tile t+1's rows 0-63 and B
-    curOff = nxtOff;
-    nxtOff = nxtOff + kRStage == kStages * kRStage ? 0 : nxtOff + kRStage;
-    dmaOff = dmaOff + kRStage == kStages * kRStage ? 0 : dmaOff + kRStage;
+    // rows 64-127 of tile t; reads tile t+1's rows 0-63 and B (wide A: tile t+1 is the other half of
+    // the same slab after an even step, the first half of the next slab after an odd one)
+    half1(p, kWideA && p == 0 ? aCur : aNxt, bNxt);
+    bCur = bNxt;
+    bNxt = next_b(bNxt);
+    bDma = next_b(bDma);
+    if (!kWideA || p == 1) {
+      aCur = aNxt;
+      aNxt = next_a(aNxt);
+      aDma = next_a(aDma);
+    }
   };
   int t = 0;
   for (; t + 1 < kTiles; t += 2) { // two steps per trip, so that the B registers' parity is a literal
@@ -564,6 +692,40 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   const bool interior = m0 + BM <= M && n0 + BN <= N; // uniform over the workgroup: nothing to mask
   if constexpr (Epi::kColumnsInRegisters) {
     const int64_t mBase = m0 + wm * WM + (lane & 15), nBase = n0 + wn * WN + (lane >> 4) * 4;
+    if constexpr (ExchangesHalfRows<Epi>::value) {
+      if (interior && N % 4 == 0) {
+        asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); // the last MFMA results are in their registers
+        const int64_t mRow = m0 + wm * WM + (lane & 7), nCol = n0 + wn * WN + ((lane >> 3) & 1) * 16 + (lane >> 4) * 4;
+#pragma unroll
+        for (int i = 0; i < FI; ++i)
+#pragma unroll
+          for (int j = 0; j < FJ; j += 2) {
+            // X = block j, Y = block j + 1.  T = X rotated by eight lanes within each row of 16; X's
+            // lanes 8-15 take Y's lanes 0-7; Y's lanes 0-7 take what X's lanes 8-15 held.  Four
+            // registers at a time, so that no DPP source was written by the three instructions before it.
+            f32x4 &X = acc[i][j], &Y = acc[i][j + 1];
+            float t0, t1, t2, t3;
+            asm volatile("v_mov_b32_dpp %8, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                         "v_mov_b32_dpp %9, %1 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                         "v_mov_b32_dpp %10, %2 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                         "v_mov_b32_dpp %11, %3 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                         "v_mov_b32_dpp %0, %4 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                         "v_mov_b32_dpp %1, %5 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                         "v_mov_b32_dpp %2, %6 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                         "v_mov_b32_dpp %3, %7 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                         "v_mov_b32_dpp %4, %8 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0x3\n\t"
+                         "v_mov_b32_dpp %5, %9 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0x3\n\t"
+                         "v_mov_b32_dpp %6, %10 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0x3\n\t"
+                         "v_mov_b32_dpp %7, %11 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0x3\n\t"
+                         "s_nop 1"
+                         : "+v"(X[0]), "+v"(X[1]), "+v"(X[2]), "+v"(X[3]), "+v"(Y[0]), "+v"(Y[1]), "+v"(Y[2]),
+                           "+v"(Y[3]), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3));
+            epi.vec4(mRow + i * 16, nCol + j * 16, N, X);
+            epi.vec4(mRow + i * 16 + 8, nCol + j * 16, N, Y);
+          }
+        return;
+      }
+    }
     if (interior) {
 #pragma unroll
       for (int i = 0; i < FI; ++i)
@@ -658,23 +820,24 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
 
 // Workgroups stride over the tiles: a launch with fewer workgroups than tiles still covers C, one
 // with more leaves the surplus nothing to do.
-template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0, bool kTail = false>
+template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0, bool kTail = false, bool kWideA = false>
 __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                            int64_t M, int64_t N, int64_t K, Epi epi, char *lds) {
   const int tilesM = int((M + BM - 1) / BM), tilesN = int((N + BN - 1) / BN);
   const int tiles = tilesM * tilesN, workgroups = gridDim.x * gridDim.y;
   for (int id = blockIdx.y * gridDim.x + blockIdx.x; id < tiles; id += workgroups) {
-    gemm_tile<T, kAT, kBT, Epi, kProbe, kTail>(A, B, M, N, K, epi, lds, tilesM, tilesN, id);
+    gemm_tile<T, kAT, kBT, Epi, kProbe, kTail, kWideA>(A, B, M, N, K, epi, lds, tilesM, tilesN, id);
     if (id + workgroups < tiles)
       __syncthreads(); // the ring is reused by this workgroup's next tile
   }
 }
 
-template <typename T, bool kAT, bool kBT, int kProbe = 0, typename Epi>
+// kWideOk: take A as 64-k-wide slabs where the shape allows (A [M,K], K a multiple of 64)
+template <typename T, bool kAT, bool kBT, int kProbe = 0, bool kWideOk = true, typename Epi>
 __device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
                                            Epi epi) {
-  // 4 stages x (256 + 256) rows x 32 k x 2 B = 128 KiB of the CU's 160 KiB LDS.
-  __shared__ __attribute__((aligned(16))) char lds[kStages * kRStage];
+  // B's four slabs (64 KiB) and A's four (64 KiB), or A's three 64-k-wide ones (96 KiB): all 160 KiB of the CU's LDS.
+  __shared__ __attribute__((aligned(16))) char lds[kLdsBytes];
   // The MFMA path wants 16-byte aligned rows in memory: K % 8 == 0 (rows of A [M,K], of B [N,K]), and a
   // row of B [K,N] (or of A [K,M] when transposed) is N (M) elements long, so those must be multiples
   // of 8 as well.  K need not fill the last 32-wide step: its copies fetch zeros beyond K.  M and N need not divide the tile: edge tiles multiply padding and store what exists.
@@ -686,7 +849,9 @@ __device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B,
   const bool tileable = M > 0 && N > 0 && K > 0 && K % 8 == 0 && (kBT || N % 8 == 0) && (!kAT || M % 8 == 0) &&
                         fitsA && fitsB &&
                         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
-  if (tileable && K % RK == 0)
+  if (!kAT && kWideOk && tileable && K % (2 * RK) == 0)
+    gemm_tiled<T, kAT, kBT, Epi, kProbe, false, !kAT && kWideOk>(A, B, M, N, K, epi, lds);
+  else if (tileable && K % RK == 0)
     gemm_tiled<T, kAT, kBT, Epi, kProbe, false>(A, B, M, N, K, epi, lds);
   else if (tileable)
     gemm_tiled<T, kAT, kBT, Epi, kProbe, true>(A, B, M, N, K, epi, lds);
