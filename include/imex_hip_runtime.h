@@ -116,7 +116,8 @@ void gpuModuleUnload(void *queue, void *module);
 void gpuMemSet32(void *queue, void *dst, unsigned int value, size_t count);
 void gpuMemSet16(void *queue, void *dst, unsigned short value, size_t count);
 
-/* ---- upstream gpu-to-llvm ABI (LevelZeroRuntimeWrappers.cpp:673-741) ---- */
+/* ---- upstream gpu-to-llvm ABI: the nine names the reference's wrapper exports
+ *      (LevelZeroRuntimeWrappers.cpp:673-741) ---- */
 void *mgpuStreamCreate(void);
 void mgpuStreamSynchronize(void *stream);
 void mgpuStreamDestroy(void *stream);
@@ -125,16 +126,17 @@ void mgpuLaunchKernel(void *kernel, size_t gridX, size_t gridY, size_t gridZ, si
                       void **params, void **extra, size_t paramsCount);
 void *mgpuMemAlloc(size_t size, void *stream, int isShared);
 void mgpuMemFree(void *stream, void *ptr);
-void mgpuMemcpy(void *dst, void *src, size_t bytes, void *stream);
-/* `count` 32-bit words of `value`.  Runs as a kernel of this library (not as a memset on the stream), so a
- * caller that captures the stream into a HIP graph gets an ordinary kernel node. */
-void mgpuMemset32(void *dst, unsigned int value, size_t count, void *stream);
-/* The 16-bit callee of the upstream gpu.memset lowering (f16 / bf16 / i16 fills); the reference
- * wrapper exports only the 32-bit one (LevelZeroRuntimeWrappers.cpp:705-711). */
-void mgpuMemset16(void *dst, unsigned short value, size_t count, void *stream);
 void *mgpuModuleLoad(const void *data, size_t dataSize);
 void *mgpuModuleGetFunction(void *module, const char *name);
 void mgpuModuleUnload(void *module);
+/* Three more callee names of upstream MLIR's gpu-to-llvm lowering (gpu.memcpy, gpu.memset of 32-bit and
+ * of 16-bit elements).  No reference line: the reference's wrapper exports the nine names above and none
+ * of these three; they are here so that host code lowered by upstream's pass finds every callee it binds.
+ * The fills run as a kernel of this library (not as a memset on the stream), so a caller that captures
+ * the stream into a HIP graph gets an ordinary kernel node; `count` is in elements. */
+void mgpuMemcpy(void *dst, void *src, size_t bytes, void *stream);
+void mgpuMemset32(void *dst, unsigned int value, size_t count, void *stream);
+void mgpuMemset16(void *dst, unsigned short value, size_t count, void *stream);
 
 /* ---- measurement helpers (no counterpart in the reference ABI; they expose
  *      the profiling loop of launchKernel, LevelZeroRuntimeWrappers.cpp:521-597,

@@ -401,18 +401,21 @@ __device__ __forceinline__ void softmax_row_in_lds(const void *in, void *out, in
     }
   }
   s = block_reduce(s, false, scratch);
+  // normalised like the other two paths: one IEEE reciprocal per row, then multiplies (an f32 rounding away
+  // from e / s at most, the same on every path, so a row's last bit does not depend on its length class)
+  const float inv = 1.0f / s;
   if (vec) {
     u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(out) + base * E::kBytes);
     for (int64_t v = threadIdx.x; v < vecs; v += kThreads) {
       float f[E::kPerVec];
 #pragma unroll
       for (int i = 0; i < E::kPerVec; ++i)
-        f[i] = rowBuf[i * vecs + v] / s;
+        f[i] = rowBuf[i * vecs + v] * inv;
       dst[v] = E::pack(f);
     }
   } else {
     for (int64_t c = threadIdx.x; c < cols; c += kThreads)
-      E::store(out, base + c, rowBuf[c] / s);
+      E::store(out, base + c, rowBuf[c] * inv);
   }
   __syncthreads(); // rowBuf is reused by the next row
 }

@@ -1,8 +1,7 @@
 // The runtime library's own device code: 32-bit and 16-bit pattern fills.
 //
-// mgpuMemset32 / mgpuMemset16 (the upstream gpu.memset lowering's callees; the 32-bit one is at
-// lib/ExecutionEngine/LEVELZERORUNTIME/LevelZeroRuntimeWrappers.cpp:705-711) and gpuMemSet32 /
-// gpuMemSet16 run these kernels instead of recording a memset on the stream, so that a caller
+// mgpuMemset32 / mgpuMemset16 (callee names of upstream MLIR's gpu.memset lowering; the reference's
+// wrapper has no counterpart) and gpuMemSet32 / gpuMemSet16 run these kernels instead of recording a memset on the stream, so that a caller
 // who captures the stream into a HIP graph gets an ordinary kernel node.
 //
 // imex_runtime_read_sweep is the second half of the profiler's cache flush: it reads a region that
