@@ -50,6 +50,13 @@
  *       WG/gemm_4kx4kx4k_transpose_a.mlir:31-55          dims = {M, N, K}
  *   imex_gemm_bf16_bias_silu_bf16  (A, B, bias, out, M:i64, N:i64, K:i64)
  *       WG/gemm_4kx4kx4k_f16_f16_f32_bias.mlir:88-113 + silu_gpu.mlir.in:3-19
+ *   imex_gemm_bf16_bias_silu_bf16_streamk  (A, B, bias, out, M:i64, N:i64, K:i64, workspace, epoch:i64, spin_limit:i64)
+ *       the same operator with the last, partial round of tiles split along K over all workgroups (no
+ *       counterpart in the reference); workspace: imexHipStreamKWorkspaceBytes(grid) bytes of device
+ *       memory, 16-byte aligned, contents irrelevant, not shared with an overlapping launch; epoch: any
+ *       value other than the one of the previous launch on that workspace; spin_limit: 0, or how many
+ *       ~1 us waits a workgroup spends on another's partial sums before computing them itself
+ *                                                          dims = {M, N, K}
  *   imex_gemm_4kx4kx4k_f16_f16_f32       (A, B, C)        dims = {}
  *   imex_gemm_4kx4kx4k_f16_f16_f32_bias  (bias, C, A, B)  dims = {}
  *   imex_gemm_4kx4kx4k_transpose_b       (A, Bt, C)       dims = {}   C += A.B^T
@@ -82,6 +89,12 @@ const void *imexHipKernelModule(const char *kernel, size_t *size);
  * -1 unknown kernel, -2 wrong number of dims or a negative / overflowing dim. */
 int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims, int ndims, size_t grid[3],
                              size_t block[3], size_t *sharedMemBytes);
+
+/* Stream-K kernels (imex_gemm_bf16_bias_silu_bf16_streamk): the most workgroups their launch shape
+ * ever asks for -- one per CU of the part -- and the workspace a launch of `workgroups` needs:
+ * 4096 bytes of flags and 256 KiB of partial sums per workgroup (64 MiB + 4 KiB at 256). */
+enum { imexHipStreamKMaxWorkgroups = 256 };
+size_t imexHipStreamKWorkspaceBytes(size_t workgroups);
 
 #ifdef __cplusplus
 }

@@ -173,6 +173,9 @@ void imexHipComputeStats(const float *values, size_t n, float *out);
 int imexHipDeviceInfo(void *queue, int *cuCount, int *clockKHz, size_t *l2Bytes, size_t *globalBytes,
                       char *name, size_t nameLen);
 
+/* The device ordinal a queue of gpuCreateStream runs on; -1 for NULL. */
+int imexHipQueueDevice(void *queue);
+
 #ifdef __cplusplus
 }
 #endif

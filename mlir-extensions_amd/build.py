@@ -7,6 +7,7 @@ Everything is compiled in-tree with explicit ``hipcc`` / ``gcc`` command lines
   lib/imex_probe.hsaco          measurement kernels (bench.py and the driver load the file; not in the catalogue)
   lib/libimex-hip-kernels.so    catalogue + the code objects embedded as blobs
   lib/libimex-hip-runtime.so    the gpu* / mgpu* runtime-wrapper ABI on HIP
+  lib/libimex-hip-ops.so        one-call entries of the K-splitting GEMM (allocating / not allocating)
   lib/libimex_runner_utils.so   _mlir_ciface_* host helpers
 
 Run as a script (``python build.py``) or call :func:`build_all`.
@@ -99,6 +100,16 @@ def build_runtime(verbose=False):
          ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib")], verbose)
 
 
+def build_ops(verbose=False):
+    """One-call operator entries: host code over the runtime ABI plus one device array, so hipcc builds it
+    (the array lives in this library's own device image)."""
+    out = os.path.join(LIB_DIR, "libimex-hip-ops.so")
+    _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "--offload-arch=gfx950",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-I" + INCLUDE_DIR,
+          os.path.join(CSRC, "ops", "GemmSplitK.hip"), "-o", out,
+          "-L" + LIB_DIR, "-limex-hip-runtime", "-limex-hip-kernels", "-Wl,-rpath,$ORIGIN"], verbose)
+
+
 def build_runner_utils(verbose=False):
     out = os.path.join(LIB_DIR, "libimex_runner_utils.so")
     _run(["g++"] + HOST_FLAGS + ["-shared", "-o", out,
@@ -126,6 +137,7 @@ def build_all(verbose=False):
     build_kernels(verbose)
     build_kernel_library(verbose)
     build_runtime(verbose)
+    build_ops(verbose)
     build_runner_utils(verbose)
     build_driver(verbose)
     build_oracle(verbose)

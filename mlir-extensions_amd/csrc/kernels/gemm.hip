@@ -49,6 +49,18 @@ extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_bf16_bias_silu_
   gemm_entry<BF16, false, false>(A, B, M, N, K, BiasSiluBF16{out, bias});
 }
 
+// The same with a workspace: the tiles that are left after the last full round of one tile per workgroup
+// have their K loops dealt out evenly over all workgroups (stream-K, gemm_tile.h).  Launch with at most
+// one workgroup per CU.  workspace: 4096 + 262144 * workgroups bytes, 16-byte aligned, not shared with a
+// launch that may overlap this one; epoch: differs from the previous launch's on the same workspace;
+// spin_limit: how long a finishing workgroup waits for the others' partial sums before it computes them
+// itself, in ~1 us units (0: about a second).  Null workspace: the kernel above.
+extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_bf16_bias_silu_bf16_streamk(
+    const uint16_t *A, const uint16_t *B, const float *bias, uint16_t *out, int64_t M, int64_t N, int64_t K,
+    void *workspace, int64_t epoch, int64_t spin_limit) {
+  gemm_entry_streamk<BF16>(A, B, M, N, K, BiasSiluBF16{out, bias}, workspace, epoch, spin_limit);
+}
+
 // C = A . B^T with B stored [N,K] (WG/gemm_4kx4kx4k_transpose_b.mlir:16,70-83: the
 // B tile is loaded k-contiguous and transposed in registers before the dpas)
 extern "C" __global__ __launch_bounds__(kThreads) void imex_gemm_f16_f16_f32_tb(const uint16_t *A, const uint16_t *Bt,

@@ -454,10 +454,31 @@ template <typename T, int kFrags> struct OperandWide {
 
 // kAT / kBT as in gemm_blocked.  A is KContig unless transposed; B is KContig only
 // when transposed.  kWideA: A's slabs are 64 k wide (A [M,K] and K a multiple of 64 only).
-// One 256 x 256 tile of C: tile number `id` of a tilesM x tilesN grid.
+// Tile number -> tile origin, XCD-aware: workgroup ids congruent mod 8 share an XCD, and the tiles they
+// take cover a compact band kGroupM tiles high, so the XCD's L2 serves few A and B panels at a time.
+struct TileOrigin {
+  int64_t m0, n0;
+};
+__device__ __forceinline__ TileOrigin tile_origin(int id, int tilesM, int tilesN) {
+  const int tiles = tilesM * tilesN;
+  int pid = id;
+  if (tiles % 8 == 0)
+    pid = (pid % 8) * (tiles / 8) + pid / 8;
+  const int group = kGroupM * tilesN;
+  const int firstM = (pid / group) * kGroupM;
+  const int groupRows = min(tilesM - firstM, kGroupM);
+  const int tileM = firstM + (pid % group) % groupRows;
+  const int tileN = (pid % group) / groupRows;
+  return TileOrigin{int64_t(tileM) * BM, int64_t(tileN) * BN};
+}
+
+// The K loop of one 256 x 256 tile of C at (m0, n0) over K-steps [ktBegin, ktEnd) (32 k each; with wide A
+// slabs both even), ADDED onto acc.  acc[i][j] is the 16 x 16 block at rows 16 i, columns 16 j of the
+// wavefront's 128 x 64 part; Epi::kColumnsInRegisters says which way round it is held (see the epilogue).
 template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0, bool kTail = false, bool kWideA = false>
-__device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, int64_t M,
-                                          int64_t N, int64_t K, Epi epi, char *lds, int tilesM, int tilesN, int id) {
+__device__ __forceinline__ void gemm_tile_mainloop(f32x4 (&acc)[FI][FJ], const uint16_t *__restrict__ A,
+                                                   const uint16_t *__restrict__ B, int64_t M, int64_t N, int64_t K,
+                                                   char *lds, int64_t m0, int64_t n0, int ktBegin, int ktEnd) {
   static_assert(FI == 8 && FJ == 4 && kWaves == 8, "written for 8 wavefronts of 8 x 4 MFMA tiles");
   static_assert(!kWideA || (!kAT && !kTail), "wide A slabs: A is [M,K] and K a multiple of 64");
   LdsChar *lds_base = (LdsChar *)lds;
@@ -466,22 +487,11 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   const int wave = tid >> 6;
   const int wm = wave / kWavesN, wn = wave % kWavesN;
 
-  // -- tile number -> tile, XCD-aware -------------------------------------------------
-  const int tiles = tilesM * tilesN;
-  int pid = id;
-  if (tiles % 8 == 0)
-    pid = (pid % 8) * (tiles / 8) + pid / 8; // ids congruent mod 8 share an XCD
-  const int group = kGroupM * tilesN;
-  const int firstM = (pid / group) * kGroupM;
-  const int groupRows = min(tilesM - firstM, kGroupM);
-  const int tileM = firstM + (pid % group) % groupRows;
-  const int tileN = (pid % group) / groupRows;
-  const int64_t m0 = int64_t(tileM) * BM, n0 = int64_t(tileN) * BN;
-
   const int waveU = __builtin_amdgcn_readfirstlane(wave);
-  const int kTiles = int((K + RK - 1) / RK);
+  const int kTiles = ktEnd - ktBegin;           // steps of this call; step t below is K-step ktBegin + t
   const int lastTile = kTiles - 1;
-  const int kRem = int(K - int64_t(lastTile) * RK); // k in the last step: 32, or 8 / 16 / 24 with kTail
+  const int lastOfK = int((K + RK - 1) / RK) - 1; // the last K-step of the whole product
+  const int kRem = int(K - int64_t(lastOfK) * RK); // k in that step: 32, or 8 / 16 / 24 with kTail
   Operand<T, kAT, FI, kTail> opA;
   OperandWide<T, FI> opAW;
   Operand<T, !kBT, FJ, kTail> opB;
@@ -494,30 +504,18 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   // Offsets below are wave-uniform byte offsets of a slab.
   constexpr int kRingA = kRingBytes;
   const int lastWide = kTiles / 2 - 1; // (kWideA: kTiles is even)
-  auto dma_a = [&](int kt, int off, int half = 0) { // narrow: K-step kt; wide: one half of 64-k slab kt
+  auto dma_a = [&](int kt, int off, int half = 0) { // narrow: step kt of this call; wide: one half of its 64-k slab kt
     if constexpr (!(kProbe & kProbeNoCopyA)) {
       if constexpr (kWideA)
-        opAW.dma(lds_base, off, kt, half);
+        opAW.dma(lds_base, off, ktBegin / 2 + kt, half);
       else
-        opA.dma(lds_base, off, kt, kTail && kt == lastTile);
+        opA.dma(lds_base, off, ktBegin + kt, kTail && ktBegin + kt == lastOfK);
     }
   };
   auto dma_b = [&](int kt, int off) {
     if constexpr (!(kProbe & kProbeNoCopyB))
-      opB.dma(lds_base, off, kt, kTail && kt == lastTile);
+      opB.dma(lds_base, off, ktBegin + kt, kTail && ktBegin + kt == lastOfK);
   };
-
-  // acc[i][j] is the 16 x 16 block at rows 16 i, columns 16 j of the wavefront's tile, held
-  // TRANSPOSED (the MFMA is given the B fragment as its first operand): lane l has row
-  // l % 16 and the four consecutive columns (l / 16) * 4 ..., which is one 16-byte store.
-  f32x4 acc[FI][FJ];
-#pragma unroll
-  for (int i = 0; i < FI; ++i)
-#pragma unroll
-    for (int j = 0; j < FJ; ++j)
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        acc[i][j][r] = 0.0f;
 
   // A step multiplies the wavefront's upper four row fragments (half 0), then the lower four
   // (half 1), each by all four B fragments.  af[h] holds half h's A fragments; bf[p] the B
@@ -676,7 +674,15 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   if (t < kTiles)
     step(0, t);
   wait_vmcnt<0>();
+}
 
+// The epilogue of a tile: what `epi` does with every element of acc that lies inside C.
+template <typename Epi, int kProbe = 0>
+__device__ __forceinline__ void gemm_tile_epilogue(f32x4 (&acc)[FI][FJ], int64_t M, int64_t N, Epi epi, int64_t m0,
+                                                   int64_t n0) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave / kWavesN, wn = wave % kWavesN;
   if constexpr (kProbe & (kProbeNoEpilogue | kProbeCopiesOnly)) {
 #pragma unroll
     for (int i = 0; i < FI; ++i)
@@ -818,6 +824,28 @@ __device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const 
   }
 }
 
+__device__ __forceinline__ void zero_accumulators(f32x4 (&acc)[FI][FJ]) {
+#pragma unroll
+  for (int i = 0; i < FI; ++i)
+#pragma unroll
+    for (int j = 0; j < FJ; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        acc[i][j][r] = 0.0f;
+}
+
+// One 256 x 256 tile of C: tile number `id` of a tilesM x tilesN grid, all of K.
+template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0, bool kTail = false, bool kWideA = false>
+__device__ __forceinline__ void gemm_tile(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, int64_t M,
+                                          int64_t N, int64_t K, Epi epi, char *lds, int tilesM, int tilesN, int id) {
+  const TileOrigin o = tile_origin(id, tilesM, tilesN);
+  f32x4 acc[FI][FJ];
+  zero_accumulators(acc);
+  gemm_tile_mainloop<T, kAT, kBT, Epi, kProbe, kTail, kWideA>(acc, A, B, M, N, K, lds, o.m0, o.n0, 0,
+                                                              int((K + RK - 1) / RK));
+  gemm_tile_epilogue<Epi, kProbe>(acc, M, N, epi, o.m0, o.n0);
+}
+
 // Workgroups stride over the tiles: a launch with fewer workgroups than tiles still covers C, one
 // with more leaves the surplus nothing to do.
 template <typename T, bool kAT, bool kBT, typename Epi, int kProbe = 0, bool kTail = false, bool kWideA = false>
@@ -832,12 +860,170 @@ __device__ __forceinline__ void gemm_tiled(const uint16_t *__restrict__ A, const
   }
 }
 
+// ---- stream-K: a tile count that does not fill the chip a whole number of times ------------------------
+// W workgroups (one per CU: the launch must not exceed the CUs, so that all of them are resident) take
+// floor(tiles / W) * W tiles whole, as above.  The K loops of the R tiles that are left -- R * K / 64
+// slabs of 64 k -- are then dealt out evenly, W consecutive ranges of slabs over the tiles laid end to end,
+// so every CU is busy for R / W of a tile's time instead of R of them for all of it.  A range touches at
+// most two tiles.  The part of a range that ends with its tile's last slab FINISHES that tile: it keeps its
+// sums in registers, adds what the earlier parts of the tile produced and runs the epilogue.  Any other part
+// is a PRODUCER: it writes its 256 x 256 partial sums (f32, 256 KiB) to the workgroup's own slot of the
+// workspace and then publishes flags[workgroup] = epoch.  A workgroup runs its producer part first and its
+// finisher part second, so a finisher only ever waits for parts that were started before it started its
+// own; the wait is bounded, and a finisher that runs out of patience computes the missing slabs itself --
+// the result is the same and the kernel always ends.
+//
+// workspace: 4096 bytes of flags (one 32-bit word per workgroup, at most 1024 workgroups), then W slots
+// of 256 KiB.  epoch: any value that differs from the one of the previous launch that used the same
+// workspace (the flags are never cleared; a stale flag cannot equal a new epoch).  Launches that share a
+// workspace must not overlap.  The sums of a tile are added in a different order than in the one-workgroup
+// form (partials, then the finisher's own), so results agree to rounding, not bit for bit.
+constexpr int kStreamKMaxWorkgroups = 1024;
+constexpr int64_t kStreamKFlagBytes = 4096, kStreamKSlotFloats = int64_t(BM) * BN;
+constexpr int kStreamKDefaultSpins = 1 << 20; // x ~1 us of sleep each: about a second
+
+// A slot holds the 32 blocks of every lane, block by block: 512 lanes x 16 bytes = 8 KiB per block, so every
+// store and load instruction moves whole lines.  Addresses are (uniform block base, pinned to scalar
+// registers by the empty asm) + (the lane's 32-bit byte offset); left alone, the compiler forms all 32
+// addresses as 64-bit vector values ahead of the K loop and spills them.
+__device__ __forceinline__ char *partial_block(const float *slot, int block) {
+  char *base = reinterpret_cast<char *>(const_cast<float *>(slot)) + block * (kThreads * 16);
+  asm volatile("" : "+s"(base));
+  return base;
+}
+__device__ __forceinline__ void store_partial(const f32x4 (&acc)[FI][FJ], float *slot) {
+  const uint32_t lane16 = threadIdx.x * 16u;
+#pragma unroll
+  for (int i = 0; i < FI; ++i)
+#pragma unroll
+    for (int j = 0; j < FJ; ++j)
+      *reinterpret_cast<f32x4 *>(partial_block(slot, i * FJ + j) + lane16) = acc[i][j];
+}
+__device__ __forceinline__ void add_partial(f32x4 (&acc)[FI][FJ], const float *slot) {
+  const uint32_t lane16 = threadIdx.x * 16u;
+#pragma unroll
+  for (int i = 0; i < FI; ++i) { // a row of blocks at a time: four loads in flight, four registers of staging
+    f32x4 v[FJ];
+#pragma unroll
+    for (int j = 0; j < FJ; ++j)
+      v[j] = *reinterpret_cast<const f32x4 *>(partial_block(slot, i * FJ + j) + lane16);
+#pragma unroll
+    for (int j = 0; j < FJ; ++j)
+      acc[i][j] += v[j];
+  }
+}
+
+template <typename T, typename Epi>
+__device__ __forceinline__ void gemm_streamk(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, int64_t M,
+                                             int64_t N, int64_t K, Epi epi, char *lds, void *workspace, int64_t epoch,
+                                             int64_t spinLimit) {
+  const int tilesM = int((M + BM - 1) / BM), tilesN = int((N + BN - 1) / BN);
+  const int tiles = tilesM * tilesN, W = gridDim.x * gridDim.y, w = blockIdx.y * gridDim.x + blockIdx.x;
+  const int kSteps = int(K / RK), full = tiles / W * W;
+  for (int id = w; id < full; id += W) {
+    gemm_tile<T, false, false, Epi, 0, false, true>(A, B, M, N, K, epi, lds, tilesM, tilesN, id);
+    __syncthreads(); // the ring is reused
+  }
+  const int R = tiles - full;
+  if (R == 0)
+    return;
+  uint32_t *flags = static_cast<uint32_t *>(workspace);
+  float *slots = reinterpret_cast<float *>(static_cast<char *>(workspace) + kStreamKFlagBytes);
+  const int64_t perTile = kSteps / 2, U = int64_t(R) * perTile; // slabs of 64 k
+  auto range_begin = [&](int q) { return int64_t(q) * U / W; };
+  const int64_t begin = range_begin(w), end = range_begin(w + 1);
+  if (begin == end)
+    return;
+  const int tFirst = int(begin / perTile), tLast = int((end - 1) / perTile);
+  const uint32_t stamp = static_cast<uint32_t>(epoch);
+  // The range's parts: the one in tile tLast when the range crosses into it (slabs from 0: a producer, unless
+  // the range happens to end with the tile), then the one in tile tFirst.  One loop around one K loop: a
+  // finisher that has waited in vain goes round once more for the slabs nobody brought.
+  const int parts = tLast != tFirst ? 2 : 1;
+  int *verdict = reinterpret_cast<int *>(lds);
+  f32x4 acc[FI][FJ];
+  for (int part = 0; part < parts; ++part) {
+    const int tile = part == parts - 1 ? tFirst : tLast;
+    const int64_t tileStart = int64_t(tile) * perTile;
+    const int64_t u0 = max(begin, tileStart) - tileStart, u1 = min(end, tileStart + perTile) - tileStart;
+    const TileOrigin o = tile_origin(full + tile, tilesM, tilesN);
+    const bool producer = u1 < perTile;
+    zero_accumulators(acc);
+    int64_t from = u0, to = u1;
+    for (bool again = true; again;) {
+      gemm_tile_mainloop<T, false, false, Epi, 0, false, true>(acc, A, B, M, N, K, lds, o.m0, o.n0, int(2 * from),
+                                                                int(2 * to));
+      __syncthreads(); // every wavefront has read its last fragments: the ring is free again
+      again = false;
+      if (producer) {
+        // Partial sums travel between workgroups on different XCDs, whose L2 caches do not see each other's
+        // lines: the producer's L2 is written back before the flag goes up (the release below, once per
+        // workgroup, after the barrier has collected every wavefront's stores), and the finisher drops what
+        // its caches hold once it has seen the flags (the acquire fence, once, outside the polling loop).
+        // Device-scope accesses alone (the sc1 bit on the slot's loads and stores, no write-back, no
+        // invalidate) were measured and gave stale partials on ordinary device allocations.
+        store_partial(acc, slots + int64_t(w) * kStreamKSlotFloats);
+        __syncthreads();
+        if (threadIdx.x == 0)
+          __hip_atomic_store(flags + w, stamp, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      } else if (from > 0) {
+        // the workgroups that hold slabs [0, u0) of this tile: from the one whose range contains the tile's
+        // first slab up to w - 1 (those with an empty range hold nothing and publish nothing)
+        int first = w;
+        while (first > 0 && range_begin(first) > tileStart)
+          --first;
+        if (threadIdx.x == 0) {
+          const int64_t limit = spinLimit > 0 ? spinLimit : kStreamKDefaultSpins;
+          int arrived = 1;
+          for (int q = first; q < w && arrived; ++q) {
+            if (range_begin(q) == range_begin(q + 1))
+              continue;
+            int64_t spins = 0;
+            while (__hip_atomic_load(flags + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != stamp) {
+              if (++spins > limit) {
+                arrived = 0;
+                break;
+              }
+              __builtin_amdgcn_s_sleep(32);
+            }
+          }
+          if (arrived)
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+          *verdict = arrived;
+        }
+        __syncthreads();
+        const int arrived = *verdict;
+        __syncthreads(); // the word is read before the ring is written again
+        if (arrived) {
+          for (int q = first; q < w; ++q)
+            if (range_begin(q) != range_begin(q + 1))
+              add_partial(acc, slots + int64_t(q) * kStreamKSlotFloats);
+        } else { // nobody came: the missing slabs, computed here, on top of what is in the registers
+          to = from;
+          from = 0;
+          again = true;
+        }
+      }
+    }
+    if (!producer)
+      gemm_tile_epilogue<Epi>(acc, M, N, epi, o.m0, o.n0);
+  }
+}
+
+// Whether gemm_streamk can take the problem: the wide-A MFMA path (see gemm_entry), a workspace, and few
+// enough workgroups for the flag words.
+__device__ __forceinline__ bool streamk_applies(const void *A, const void *B, int64_t M, int64_t N, int64_t K,
+                                                const void *workspace) {
+  constexpr int64_t kMaxBytes = int64_t(1) << 31, kMaxRow = int64_t(1) << 22;
+  return workspace != nullptr && M > 0 && N > 0 && K > 0 && K % (2 * RK) == 0 && N % 8 == 0 && K < kMaxRow &&
+         K * N * 2 < kMaxBytes && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 &&
+         (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 && int(gridDim.x * gridDim.y) <= kStreamKMaxWorkgroups;
+}
+
 // kWideOk: take A as 64-k-wide slabs where the shape allows (A [M,K], K a multiple of 64)
 template <typename T, bool kAT, bool kBT, int kProbe = 0, bool kWideOk = true, typename Epi>
-__device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
-                                           Epi epi) {
-  // B's four slabs (64 KiB) and A's four (64 KiB), or A's three 64-k-wide ones (96 KiB): all 160 KiB of the CU's LDS.
-  __shared__ __attribute__((aligned(16))) char lds[kLdsBytes];
+__device__ __forceinline__ void gemm_dispatch(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
+                                              Epi epi, char *lds) {
   // The MFMA path wants 16-byte aligned rows in memory: K % 8 == 0 (rows of A [M,K], of B [N,K]), and a
   // row of B [K,N] (or of A [K,M] when transposed) is N (M) elements long, so those must be multiples
   // of 8 as well.  K need not fill the last 32-wide step: its copies fetch zeros beyond K.  M and N need not divide the tile: edge tiles multiply padding and store what exists.
@@ -857,6 +1043,26 @@ __device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B,
     gemm_tiled<T, kAT, kBT, Epi, kProbe, true>(A, B, M, N, K, epi, lds);
   else
     gemm_blocked<T, kAT, kBT, Epi>(A, B, M, N, K, epi, lds);
+}
+
+template <typename T, bool kAT, bool kBT, int kProbe = 0, bool kWideOk = true, typename Epi>
+__device__ __forceinline__ void gemm_entry(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N, int64_t K,
+                                           Epi epi) {
+  // B's four slabs (64 KiB) and A's four (64 KiB), or A's three 64-k-wide ones (96 KiB): all 160 KiB of the CU's LDS.
+  __shared__ __attribute__((aligned(16))) char lds[kLdsBytes];
+  gemm_dispatch<T, kAT, kBT, kProbe, kWideOk>(A, B, M, N, K, epi, lds);
+}
+
+// Entry with a workspace: stream-K where it applies, otherwise exactly gemm_entry.
+template <typename T, typename Epi>
+__device__ __forceinline__ void gemm_entry_streamk(const uint16_t *A, const uint16_t *B, int64_t M, int64_t N,
+                                                   int64_t K, Epi epi, void *workspace, int64_t epoch,
+                                                   int64_t spinLimit) {
+  __shared__ __attribute__((aligned(16))) char lds[kLdsBytes];
+  if (streamk_applies(A, B, M, N, K, workspace))
+    gemm_streamk<T, Epi>(A, B, M, N, K, epi, lds, workspace, epoch, spinLimit);
+  else
+    gemm_dispatch<T, false, false>(A, B, M, N, K, epi, lds);
 }
 
 } // namespace imexhip_gemm

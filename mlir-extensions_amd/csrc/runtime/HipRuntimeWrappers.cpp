@@ -784,6 +784,8 @@ extern "C" void imexHipComputeStats(const float *values, size_t n, float *out) {
   out[8] = s.middleThirdAvg;
 }
 
+extern "C" int imexHipQueueDevice(void *queue) { return queue ? asQueue(queue)->device : -1; }
+
 extern "C" int imexHipDeviceInfo(void *queue, int *cuCount, int *clockKHz, size_t *l2Bytes,
                                  size_t *globalBytes, char *name, size_t nameLen) {
   int device = queue ? asQueue(queue)->device : defaultDeviceOrdinal();

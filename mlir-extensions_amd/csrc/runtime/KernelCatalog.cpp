@@ -28,7 +28,7 @@ extern const unsigned char imex_blob_attention[], imex_blob_attention_end[];
 namespace {
 
 enum class Module { Eltwise, Softmax, Reduce, Transpose, Gemm, Fusion, Attention };
-enum class Shape { Eltwise32, Eltwise16, Fusion32, Fusion16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, ReduceOuter16, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, ColumnThreads16, Attention };
+enum class Shape { Eltwise32, Eltwise16, Fusion32, Fusion16, SoftmaxRows32, SoftmaxRows16, RowSum, ReduceOuter, ReduceOuter16, Transpose2D32, Transpose2D16, Transpose3D32, Transpose3D16, Gemm, GemmStreamK, GemmTA, GemmTB, GemmFixed4k, ColumnThreads, ColumnThreads16, Attention };
 
 struct Entry {
   const char *name;
@@ -84,6 +84,9 @@ const Entry kEntries[] = {
     {"imex_gemm_f16_f16_f16", "(A: f16*, B: f16*, C: f16*, M: i64, N: i64, K: i64)", Module::Gemm, Shape::Gemm, 3},
     {"imex_gemm_bf16_bias_silu_bf16", "(A: bf16*, B: bf16*, bias: f32*, out: bf16*, M: i64, N: i64, K: i64)",
      Module::Gemm, Shape::Gemm, 3},
+    {"imex_gemm_bf16_bias_silu_bf16_streamk",
+     "(A: bf16*, B: bf16*, bias: f32*, out: bf16*, M: i64, N: i64, K: i64, workspace: i8*, epoch: i64, spin_limit: i64)",
+     Module::Gemm, Shape::GemmStreamK, 3},
     {"imex_gemm_f16_f16_f32_tb", "(A: f16*, Bt: f16* [N,K], C: f32*, M: i64, N: i64, K: i64)", Module::Gemm,
      Shape::GemmTB, 3},
     {"imex_gemm_f16_f16_f32_ta", "(At: f16* [K,M], B: f16*, C: f32*, M: i64, N: i64, K: i64)", Module::Gemm,
@@ -137,6 +140,8 @@ extern "C" const void *imexHipKernelModule(const char *kernel, size_t *size) {
     *size = static_cast<size_t>(end - begin);
   return begin;
 }
+
+extern "C" size_t imexHipStreamKWorkspaceBytes(size_t workgroups) { return 4096 + (size_t(256) * 256 * 4) * workgroups; }
 
 extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims, int ndims, size_t grid[3],
                                         size_t block[3], size_t *sharedMemBytes) {
@@ -290,6 +295,19 @@ extern "C" int imexHipKernelLaunchShape(const char *kernel, const int64_t *dims,
     const bool tileable = M > 0 && N > 0 && K > 0 && K % 8 == 0 && rowsA && rowsB && fitsA && fitsB;
     block[0] = 512;
     grid[0] = tileable ? ceilDiv(M, 256) * ceilDiv(N, 256) : ceilDiv(M, 128) * ceilDiv(N, 128);
+    break;
+  }
+  case Shape::GemmStreamK: {
+    // One workgroup per CU at most (256 on this part): the kernel's finishing workgroups wait for partial sums
+    // of others, which have to be resident.  A problem with fewer tiles than CUs still gets more workgroups
+    // than tiles -- its K loops are split -- as long as each one has 1024 k or more to do.
+    const int64_t M = dims[0], N = dims[1], K = dims[2];
+    const bool streams = M > 0 && N > 0 && K > 0 && K % 64 == 0 && N % 8 == 0;
+    const size_t tiles = ceilDiv(M, 256) * ceilDiv(N, 256);
+    const size_t shares = K >= 2048 ? static_cast<size_t>(K / 1024) : 1;
+    block[0] = 512;
+    grid[0] = !streams ? (K % 8 == 0 && N % 8 == 0 ? tiles : ceilDiv(M, 128) * ceilDiv(N, 128))
+                       : std::min<size_t>(imexHipStreamKMaxWorkgroups, tiles * shares);
     break;
   }
   case Shape::GemmFixed4k: // the reference's own launch: blocks (16,16,1), threads (512,1,1)

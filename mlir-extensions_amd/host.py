@@ -76,6 +76,12 @@ _RUNTIME_SYMBOLS = {
     "imexHipComputeStats": (None, [C.POINTER(C.c_float), C.c_size_t, C.POINTER(C.c_float)]),
     "imexHipDeviceInfo": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_size_t),
                                     C.POINTER(C.c_size_t), C.c_char_p, C.c_size_t]),
+    "imexHipQueueDevice": (C.c_int, [C.c_void_p]),
+}
+
+_OPS_SYMBOLS = {
+    "imexHipGemmBiasSiluBf16SplitK": (C.c_int, [C.c_void_p] * 5 + [C.c_int64] * 3),
+    "imexHipOpsLastError": (C.c_char_p, []),
 }
 
 _KERNEL_SYMBOLS = {
@@ -85,6 +91,7 @@ _KERNEL_SYMBOLS = {
     "imexHipKernelModule": (C.c_void_p, [C.c_char_p, C.POINTER(C.c_size_t)]),
     "imexHipKernelLaunchShape": (C.c_int, [C.c_char_p, C.POINTER(C.c_int64), C.c_int, C.POINTER(C.c_size_t),
                                            C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "imexHipStreamKWorkspaceBytes": (C.c_size_t, [C.c_size_t]),
 }
 
 _RUNNER_UTILS_SYMBOLS = [
@@ -130,6 +137,21 @@ def kernels():
         _bind(lib, _KERNEL_SYMBOLS)
         _kernels = lib
     return _kernels
+
+
+_ops = None
+
+
+def ops():
+    """libimex-hip-ops.so: the one-call operator entries (include/imex_hip_ops.h)."""
+    global _ops
+    if _ops is None:
+        runtime()
+        kernels()
+        lib = _load("libimex-hip-ops.so")
+        _bind(lib, _OPS_SYMBOLS)
+        _ops = lib
+    return _ops
 
 
 def runner_utils():
@@ -571,18 +593,31 @@ def gemm(stream, a, b, c=None, ab_dtype="f16", out_dtype="f32", trans_a=False, t
             stream.free(p)
 
 
-def gemm_bias_silu(stream, a, b, bias):
-    """out = bf16(silu(A.B + bias[n])) with bf16 A, B and f32 bias."""
+_streamk_epoch = [0]
+
+
+def gemm_bias_silu(stream, a, b, bias, streamk=False, grid=None, spin_limit=0):
+    """out = bf16(silu(A.B + bias[n])) with bf16 A, B and f32 bias.  streamk: the kernel that splits the
+    last, partial round of tiles along K over all workgroups (a workspace is allocated for the call)."""
     _check(a, "bf16")
     _check(b, "bf16")
     M, K = a.shape
     _, N = b.shape
     d_a, d_b, d_bias = stream.to_device(a), stream.to_device(b), stream.to_device(bias.astype(np.float32))
     d_o = stream.alloc(max(M * N, 1) * 2)
+    d_ws = None
     try:
-        stream.launch("imex_gemm_bf16_bias_silu_bf16", [M, N, K], [d_a, d_b, d_bias, d_o, M, N, K])
+        if streamk:
+            name = "imex_gemm_bf16_bias_silu_bf16_streamk"
+            g = grid if grid is not None else launch_shape(name, [M, N, K])[0]
+            d_ws = stream.alloc(kernels().imexHipStreamKWorkspaceBytes(g[0] * g[1] * g[2]))
+            _streamk_epoch[0] += 1
+            stream.launch(name, [M, N, K], [d_a, d_b, d_bias, d_o, M, N, K, d_ws, _streamk_epoch[0], spin_limit], grid=grid)
+        else:
+            stream.launch("imex_gemm_bf16_bias_silu_bf16", [M, N, K], [d_a, d_b, d_bias, d_o, M, N, K], grid=grid)
         stream.wait()
         return stream.from_device(d_o, (M, N), np.uint16)
     finally:
-        for p in (d_a, d_b, d_bias, d_o):
-            stream.free(p)
+        for p in (d_a, d_b, d_bias, d_o, d_ws):
+            if p is not None:
+                stream.free(p)

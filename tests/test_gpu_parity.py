@@ -1040,6 +1040,91 @@ def test_gemm_config_mlp_bf16_bias_silu(host, orc, stream):
     assert np.all(d <= 2.0 ** -7 * np.abs(want) + 1e-6), "fused epilogue differs at %s" % (np.argwhere(d > 2.0 ** -7 * np.abs(want) + 1e-6)[:4],)
 
 
+def _streamk_against_plain(host, orc, a, b, bias, stream, **kw):
+    """The stream-K kernel against the one-workgroup-per-tile kernel on the same operands: the f32 sums
+    of a split tile are added in another order (partials, then the finisher's own), so the bf16 results
+    agree to a rounding step of the output type, and mostly bit for bit."""
+    plain = host.gemm_bias_silu(stream, a, b, bias)
+    got = host.gemm_bias_silu(stream, a, b, bias, streamk=True, **kw)
+    p, g = orc.bfloat_to_float(plain), orc.bfloat_to_float(got)
+    assert np.array_equal(np.isnan(p), np.isnan(g))
+    d = np.abs(p - g)
+    # a step of the output type, plus the f32 rounding of a sum of K products where the sum nearly cancels
+    bad = d > 2.0 ** -7 * np.abs(p) + 1e-4
+    assert not bad.any(), (np.argwhere(bad)[:4], p[bad][:4], g[bad][:4])
+    return float(np.mean(plain == got))
+
+
+@pytest.mark.parametrize("M,N,K,grid", [
+    (512, 768, 256, None),        # 6 tiles, 4 slabs of 64 k each: one workgroup per tile, nothing to split
+    (512, 768, 4096, None),       # 6 tiles over 24 workgroups: every tile split four ways
+    (1024, 1280, 2048, (7, 1, 1)),    # 20 tiles on 7 workgroups: two full rounds, 6 tiles dealt out over 7
+    (1000, 520, 1024, (5, 1, 1)),     # ragged edge tiles, 12 tiles on 5 workgroups
+    (256, 256, 8192, (16, 1, 1)),     # one tile, sixteen parts: a finisher with fifteen partners
+    (300, 264, 192, (64, 1, 1)),      # more workgroups than slabs: most ranges are empty
+    (512, 512, 96, (3, 1, 1)),        # K % 64 != 0: the kernel takes the ordinary path and ignores the workspace
+])
+def test_gemm_streamk_small_shapes(host, orc, stream, M, N, K, grid):
+    say("stream-K %dx%dx%d grid %s" % (M, N, K, grid))
+    a = orc.fill_normal(M * K, "bf16", 31, 0.0, 1.0).reshape(M, K)
+    b = orc.fill_normal(K * N, "bf16", 32, 0.0, 0.05).reshape(K, N)
+    bias = orc.fill_normal(N, "f32", 33, 0.0, 0.1)
+    _streamk_against_plain(host, orc, a, b, bias, stream, grid=grid)
+    # integer operands: every order of additions gives the same f32 sums, so the two kernels agree bit for bit
+    a = orc.fill_int(M * K, "bf16", 34, -2, 2).reshape(M, K)
+    b = orc.fill_int(K * N, "bf16", 35, -2, 2).reshape(K, N)
+    assert _streamk_against_plain(host, orc, a, b, np.zeros(N, np.float32), stream, grid=grid) == 1.0
+    # ... and twice in a row on one workspace with consecutive epochs (flags of the first launch are stale)
+    assert _streamk_against_plain(host, orc, a, b, np.zeros(N, np.float32), stream, grid=grid) == 1.0
+
+
+def test_gemm_streamk_impatient_finisher(host, orc, stream):
+    """A finishing workgroup that is allowed a single look at its partners' flags mostly finds them unset
+    and computes the missing slabs itself: the same results, and the kernel ends either way."""
+    M, N, K = 768, 512, 4096
+    a = orc.fill_int(M * K, "bf16", 36, -2, 2).reshape(M, K)
+    b = orc.fill_int(K * N, "bf16", 37, -2, 2).reshape(K, N)
+    bias = orc.fill_normal(N, "f32", 38, 0.0, 0.1)
+    for grid in ((24, 1, 1), (5, 1, 1)):
+        assert _streamk_against_plain(host, orc, a, b, bias, stream, grid=grid, spin_limit=1) == 1.0
+
+
+def test_gemm_streamk_config_mlp(host, orc, stream):
+    """The MLP configuration: 688 tiles on 256 workgroups, two full rounds and 176 tiles dealt out."""
+    M, K, N = 4096, 4096, 11008
+    a = orc.fill_normal(M * K, "bf16", 20248, 0.0, 1.0).reshape(M, K)
+    b = orc.fill_normal(K * N, "bf16", 20249, 0.0, 0.02).reshape(K, N)
+    bias = orc.fill_normal(N, "f32", 20250, 0.0, 0.1)
+    assert host.launch_shape("imex_gemm_bf16_bias_silu_bf16_streamk", [M, N, K])[0] == (256, 1, 1)
+    same = _streamk_against_plain(host, orc, a, b, bias, stream)
+    say("stream-K MLP: %.4f of the outputs bit-identical to the plain kernel" % same)
+    assert same > 0.95
+
+
+def test_gemm_split_k_operator_entry(host, orc, stream):
+    """imexHipGemmBiasSiluBf16SplitK (include/imex_hip_ops.h): the K-splitting kernel behind one call that
+    sizes, allocates and stamps the workspace itself -- a few-tile, deep-K problem, then a larger one (the
+    workspace grows), then the first again; each against the one-workgroup-per-tile kernel."""
+    ops = host.ops()
+    for M, N, K in ((512, 512, 8192), (1024, 1280, 4096), (512, 512, 8192)):
+        say("split-K operator entry %dx%dx%d" % (M, N, K))
+        a = orc.fill_int(M * K, "bf16", 71, -2, 2).reshape(M, K)
+        b = orc.fill_int(K * N, "bf16", 72, -2, 2).reshape(K, N)
+        bias = orc.fill_normal(N, "f32", 73, 0.0, 0.1)
+        d_a, d_b, d_bias = stream.to_device(a), stream.to_device(b), stream.to_device(bias)
+        d_o = stream.to_device(np.full((M, N), 0x7FC1, np.uint16))
+        rc = ops.imexHipGemmBiasSiluBf16SplitK(stream.handle, int(d_a), int(d_b), int(d_bias), int(d_o), M, N, K)
+        assert rc == 0, ops.imexHipOpsLastError()
+        stream.wait()
+        got = stream.from_device(d_o, (M, N), np.uint16)
+        for p in (d_a, d_b, d_bias, d_o):
+            stream.free(p)
+        # integer operands: the f32 sums are exact in any order, so the two kernels agree bit for bit
+        assert np.array_equal(got, host.gemm_bias_silu(stream, a, b, bias)), (M, N, K)
+    assert ops.imexHipGemmBiasSiluBf16SplitK(None, None, None, None, None, 256, 256, 64) == -1
+    assert b"queue" in ops.imexHipOpsLastError()
+
+
 def test_gemm_reference_bias_kernel_4096(host, orc, stream):
     """WG/gemm_4kx4kx4k_f16_f16_f32_bias.mlir:77-116: kernel arguments (bias, C, A, B), grid 16 x 16,
     C = bias[n] + (C + A.B); checked as the test itself does (:160-172): the f32 GEMM onto the initial C,

@@ -51,6 +51,17 @@ def test_kernel_library_exports_and_catalogue(host):
     assert k.imexHipKernelModule(b"no_such_kernel", None) is None
 
 
+def test_ops_library_exports_every_declared_symbol(host):
+    ops = host.ops()
+    names = declared_functions("imex_hip_ops.h")
+    assert "imexHipGemmBiasSiluBf16SplitK" in names and len(names) == 2
+    for n in names:
+        assert getattr(ops, n) is not None, n
+    assert set(names) == set(host._OPS_SYMBOLS)
+    # no compute without a GPU: only what needs none
+    assert ops.imexHipOpsLastError() == b""
+
+
 def test_runner_utils_exports(host):
     ru = host.runner_utils()
     for n in declared_functions("imex_runner_utils.h"):
