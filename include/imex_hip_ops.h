@@ -23,12 +23,31 @@
 extern "C" {
 #endif
 
+/* Once per device before the first imexHipGemmBiasSiluBf16SplitKNoAlloc on it (further calls do nothing):
+ * loads the code object, resolves the kernel and this device's copy of the library's fixed workspace.
+ * May allocate (the HIP runtime places the code object in device memory). */
+int imexHipOpsInit(void *queue);
+
 /* out = bf16(silu(A.B + bias[n])) with the K loops split over the chip's CUs.  The workspace
  * (imexHipStreamKWorkspaceBytes of the launch's workgroups: at most 64 MiB + 4 KiB) is allocated by the
  * library on the first call on a device and kept for the life of the process.  Calls on one device that may
  * overlap in time (different queues) must not be made: they would share the workspace. */
 int imexHipGemmBiasSiluBf16SplitK(void *queue, const void *A, const void *B, const void *bias, void *out,
                                   int64_t M, int64_t N, int64_t K);
+
+/* The same operator for callers that cannot allocate device memory at the point of the call -- code under
+ * HIP graph capture, tight serving loops, harnesses that forbid it.  No counterpart in the reference.
+ * Allocates nothing and calls nothing that allocates: the workspace is a fixed array of 64 MiB + 4 KiB in
+ * the library's own device image (every GPU the library runs on holds one until the process ends), which
+ * is the most the kernel's launch shape ever needs; a launch that would need more is refused (-3).
+ * Requires imexHipOpsInit on the queue's device (-2 otherwise).  All calls on one GPU share that array:
+ * calls that overlap in time race, and nothing in it has to be cleared between calls (the flags in it are
+ * stamped with a per-device launch counter). */
+int imexHipGemmBiasSiluBf16SplitKNoAlloc(void *queue, const void *A, const void *B, const void *bias,
+                                         void *out, int64_t M, int64_t N, int64_t K);
+
+/* The bytes of the fixed workspace behind the NoAlloc entry. */
+size_t imexHipOpsFixedWorkspaceBytes(void);
 
 /* What went wrong in the calling thread's last failing call ("" if none has failed). */
 const char *imexHipOpsLastError(void);

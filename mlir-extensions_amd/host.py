@@ -80,7 +80,10 @@ _RUNTIME_SYMBOLS = {
 }
 
 _OPS_SYMBOLS = {
+    "imexHipOpsInit": (C.c_int, [C.c_void_p]),
     "imexHipGemmBiasSiluBf16SplitK": (C.c_int, [C.c_void_p] * 5 + [C.c_int64] * 3),
+    "imexHipGemmBiasSiluBf16SplitKNoAlloc": (C.c_int, [C.c_void_p] * 5 + [C.c_int64] * 3),
+    "imexHipOpsFixedWorkspaceBytes": (C.c_size_t, []),
     "imexHipOpsLastError": (C.c_char_p, []),
 }
 

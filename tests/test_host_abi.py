@@ -54,11 +54,12 @@ def test_kernel_library_exports_and_catalogue(host):
 def test_ops_library_exports_every_declared_symbol(host):
     ops = host.ops()
     names = declared_functions("imex_hip_ops.h")
-    assert "imexHipGemmBiasSiluBf16SplitK" in names and len(names) == 2
+    assert "imexHipGemmBiasSiluBf16SplitKNoAlloc" in names and len(names) == 5
     for n in names:
         assert getattr(ops, n) is not None, n
     assert set(names) == set(host._OPS_SYMBOLS)
     # no compute without a GPU: only what needs none
+    assert ops.imexHipOpsFixedWorkspaceBytes() == host.kernels().imexHipStreamKWorkspaceBytes(256)
     assert ops.imexHipOpsLastError() == b""
 
 
