@@ -40,6 +40,8 @@ int imexHipGemmBiasSiluBf16SplitK(void *queue, const void *A, const void *B, con
  * Allocates nothing and calls nothing that allocates: the workspace is a fixed array of 64 MiB + 4 KiB in
  * the library's own device image (every GPU the library runs on holds one until the process ends), which
  * is the most the kernel's launch shape ever needs; a launch that would need more is refused (-3).
+ * (With the runtime's profiling mode switched off, as it is by default: IMEX_ENABLE_PROFILING makes every
+ * gpuLaunchKernel time its kernel first, and that loop allocates.)
  * Requires imexHipOpsInit on the queue's device (-2 otherwise).  All calls on one GPU share that array:
  * calls that overlap in time race, and nothing in it has to be cleared between calls (the flags in it are
  * stamped with a per-device launch counter). */

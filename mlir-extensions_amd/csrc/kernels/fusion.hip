@@ -296,7 +296,7 @@ __device__ __forceinline__ void input_fusion_cols(const void *__restrict__ a, co
 constexpr int kStreamWorkers = 512, kStreamThreads = kStreamWorkers + 64;
 constexpr int kNarrowWorkers = 256, kNarrowThreads = kNarrowWorkers + 64;
 constexpr int kStreamTileElems = 8192;
-constexpr int kStreamTileFloats = 64 * (128 + 4); // the largest padded tile: 64 columns of 128 rows
+constexpr int kStreamTileFloats = 64 * (128 + 16); // the largest padded tile: 64 columns of 128 rows
 constexpr int64_t kStreamFromRows = 2048;
 
 // kLanesPerRow worker lanes cover a row segment, each with one 16-byte vector (kVec) or one element; an access
@@ -310,22 +310,20 @@ template <Dt D, int kLanesPerRow, int kWorkers, int kTilePassesT, int kGroupTile
   static constexpr int kRowsPerPass = kWorkers / kLanesPerRow;
   static constexpr int kTileRows = kTilePasses * kRowsPerPass;
   static constexpr int kGroupPasses = kTilePasses * kGroupTiles;
-  // A tile lies in LDS COLUMN by column, kTileRows + 4 floats apart: the adder reads four consecutive rows of its
-  // column with one 128-bit access, and the pad puts the columns of neighbouring lanes into different banks.
-  // Row r of column c sits at position r ^ row_swizzle(c), a multiple of 8 below 32 (blocks of eight rows
-  // trade places; the adder's groups of four rows stay together).  With a pitch that is 4 modulo 64, the
-  // column groups a worker wavefront writes with one instruction (eight groups, eight rows each) would
-  // otherwise share banks -- every write two-way conflicted for f32, four-way for 16-bit elements.  The
-  // swizzle is chosen so that those writes AND the adder's 128-bit reads (one lane per column; the LDS
-  // serves such reads sixteen lanes at a time: 0-3 with 12-15, 20-23 and 24-27, ...) touch every bank once:
-  // 8 x the parity of the column's group of four among eight, + 16 for columns 32-63.
-  static constexpr int kColPitch = kTileRows + 4;
-  static __device__ __forceinline__ int row_swizzle(int col) {
-    const int g = (col >> 2) & 7;
-    return (((g ^ (g >> 1) ^ (g >> 2)) & 1) << 3) | (((col >> 5) & 1) << 4);
-  }
+  // A tile lies in LDS COLUMN by column, kTileRows + 16 floats apart, and row r of column c sits at position
+  // r ^ row_swizzle(c), a multiple of 4 below 32: blocks of four rows trade places inside their block of 32,
+  // so the adder still reads four consecutive rows of its column with one 128-bit access.  Pitch and swizzle
+  // follow from how the LDS serves the two kinds of access (measured with two-lane probes): a 32-bit write is
+  // served 32 lanes at a time (0-31, 32-63) over banks that repeat every 32 words; a 128-bit read sixteen
+  // lanes at a time (0-3 with 12-15, 20-23 and 24-27; 4-11 with 16-19 and 28-31; the same + 32) over banks
+  // that repeat every 64 words.  A worker half-wavefront writes four rows of eight column groups with one
+  // instruction: the pitch (16 modulo 32 words) puts odd and even groups 16 banks apart, the swizzle
+  // 4 x (group index) spreads the four groups of each kind over the four 4-bank blocks.  The adder's sixteen
+  // lanes then read sixteen different 16-byte bank groups for every row block.
+  static constexpr int kColPitch = kTileRows + 16;
+  static __device__ __forceinline__ int row_swizzle(int col) { return 4 * ((col / kPer) & 7); }
   static constexpr int kTileFloats = kCols * kColPitch;
-  static_assert(kTileRows % 32 == 0 && kTileFloats <= kStreamTileFloats, "the LDS tiles are sized for 8448 floats");
+  static_assert(kTileRows % 32 == 0 && kTileFloats <= kStreamTileFloats, "the LDS tiles are sized for 9216 floats");
 };
 // wide: 128-byte row segments, 8192-element tiles (256 rows of 32 f32, 128 rows of 64 16-bit columns)
 template <Dt D>
@@ -344,7 +342,7 @@ __device__ __forceinline__ bool input_fusion_narrow(int64_t cols) { return cols 
 // acc + c[0] + c[1] + ... + c[n-1], added in that order, for a column c of kTileRows consecutive floats
 // (16-byte aligned, all of them readable): sixteen rows arrive as four 128-bit LDS reads while the previous
 // sixteen are added, so the adder issues 1.25 instructions per row.
-// swz: row r is kept at position r ^ swz (a multiple of 8 below 32: blocks of eight rows trade places).
+// swz: row r is kept at position r ^ swz (a multiple of 4 below 32: blocks of four rows trade places).
 template <int kTileRows>
 __device__ __forceinline__ float add_column_in_row_order(float acc, const float *c, int n, int swz = 0) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));

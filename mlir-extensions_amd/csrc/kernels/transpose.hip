@@ -188,7 +188,10 @@ __device__ __forceinline__ void tile16_fast(const uint16_t *__restrict__ in, uin
 // barrier per quarter is enough: when a wavefront writes quarter q + 2 into an image, every wavefront has
 // passed the barrier of quarter q + 1 and with it its last read of quarter q.  Loads and stores are
 // unconditional straight-line code, so the waits are exact counts ("all but the 24, 16, 8 youngest").
-// LDS image T[64 columns][256 rows]: group g (eight rows) of column c at position g ^ (2 (c / 8)).
+// LDS image T[64 columns][256 rows]: group g (eight rows) of column c at position g ^ (c / 8).  A 128-bit LDS
+// write is served eight consecutive lanes at a time over 128 bytes of banks: those eight lanes are the eight
+// column blocks of one row block, whose positions differ in their low three bits.  A 128-bit read is served
+// sixteen lanes at a time over 256 bytes of banks: one output row's groups, sixteen different positions.
 __device__ __forceinline__ void tile16_quarters(const uint16_t *__restrict__ in, uint16_t *__restrict__ out,
                                                 const View &v, int64_t r0, int64_t c0, u32x4 *lds) {
   constexpr int G = 32;            // 16-byte groups per LDS row (256 rows of the tile)
@@ -202,7 +205,7 @@ __device__ __forceinline__ void tile16_quarters(const uint16_t *__restrict__ in,
 #pragma unroll
     for (int j = 0; j < 8; ++j)
       x[q][j] = load128<true>(reinterpret_cast<const u32x4 *>(src + j * v.ldIn + q * 64));
-  const int pos = b ^ (2 * cg);
+  const int pos = b ^ cg;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     u32x4 *img = lds + (q & 1) * kImage;
@@ -223,7 +226,7 @@ __device__ __forceinline__ void tile16_quarters(const uint16_t *__restrict__ in,
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
       const int c = cc + 8 * p; // output row within the quarter
-      y[p] = img[c * G + (g ^ (2 * (c >> 3)))];
+      y[p] = img[c * G + (g ^ (c >> 3))];
     }
 #pragma unroll
     for (int p = 0; p < 8; ++p)
