@@ -314,6 +314,39 @@ def measure_rotating(host, stream, w, passes):
     return ms, copies
 
 
+def measure_split_k(stream, host):
+    """out = bf16(silu(A.B + bias)) through the plain kernel and through the K-splitting operator entry
+    (imexHipGemmBiasSiluBf16SplitK of libimex-hip-ops.so), same buffers back to back: ms per launch for the MLP
+    shape (many tiles: the plain kernel is the faster one) and for shapes with few tiles and a deep K loop (where
+    splitting K is what fills the chip).  Zero-filled operands: this compares schedules, not clocks."""
+    ops = host.ops()
+    if ops.imexHipOpsInit(stream.handle) != 0:
+        raise RuntimeError("imexHipOpsInit: %s" % ops.imexHipOpsLastError().decode())
+    out = {}
+    for M, N, K in ((4096, 11008, 4096), (2048, 2048, 4096), (1024, 1024, 8192), (512, 512, 16384)):
+        a, b, bias, o = stream.alloc(M * K * 2), stream.alloc(K * N * 2), stream.alloc(N * 4), stream.alloc(M * N * 2)
+        for ptr, n in ((a, M * K // 2), (b, K * N // 2), (bias, N)):
+            stream.memset(ptr, 0, n, bits=32)
+        plain = stream.profile("imex_gemm_bf16_bias_silu_bf16", [M, N, K], [a, b, bias, o, M, N, K],
+                               warmups=50, rounds=200, mode=1)[0] / 200
+
+        def split():
+            if ops.imexHipGemmBiasSiluBf16SplitK(stream.handle, int(a), int(b), int(bias), int(o), M, N, K) != 0:
+                raise RuntimeError(ops.imexHipOpsLastError().decode())
+        for _ in range(50):
+            split()
+        stream.wait()
+        ev0 = stream.timestamp()
+        for _ in range(200):
+            split()
+        ev1 = stream.timestamp()
+        stream.wait()
+        out["%dx%dx%d" % (M, N, K)] = {"plain_ms": round(plain, 5), "split_k_ms": round(stream.elapsed_ms(ev0, ev1) / 200, 5)}
+        for ptr in (a, b, bias, o):
+            stream.free(ptr)
+    return out
+
+
 def measure_reference_suite(stream):
     """Every shape and dtype the reference's benchmark suite instantiates (README.md:330-335, benchmarks/*/
     *.shapes.in, *.dtypes.in) plus the two fused chains at their size (512x1024): microseconds per launch over 200
@@ -679,6 +712,8 @@ def main():
     if args.suite:
         result["reference_suite_us_per_launch"] = measure_reference_suite(stream)
         log("reference benchmark suite: %d shapes timed" % len(result["reference_suite_us_per_launch"]))
+        result["gemm_bias_silu_split_k_ms_per_launch_MxNxK"] = measure_split_k(stream, host)
+        log("split-K operator entry against the plain kernel: %s" % result["gemm_bias_silu_split_k_ms_per_launch_MxNxK"])
 
     for w in workloads:
         for p in w.buffers:

@@ -15,6 +15,7 @@
 //
 //   imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--rotate S] [--grid G] [--launch-only N] <workload>...
 //   imex-hip-bench --list
+//   imex-hip-bench --lds-service       (LDS lane-grouping / bank-period probe, for a bank-conflict counter run)
 //   imex-hip-bench [-l] --report report.txt <workload>...|all|operators
 //
 //   --report FILE  bench_imex's outer loop (bench_imex.in:72-91): one child process per workload,
@@ -323,6 +324,60 @@ struct Options {
   bool flush = false, zeros = false;
 };
 
+// The measurement kernels' code object, read once and kept for the life of the process (the runtime caches
+// modules by address); empty if the file is not beside this program.
+const std::vector<char> &probeImage() {
+  static std::vector<char> image;
+  if (image.empty()) {
+    const std::string path = programDir() + "/imex_probe.hsaco";
+    if (FILE *f = fopen(path.c_str(), "rb")) {
+      char buf[65536];
+      for (size_t n; (n = fread(buf, 1, sizeof buf, f)) > 0;)
+        image.insert(image.end(), buf, buf + n);
+      fclose(f);
+    }
+  }
+  return image;
+}
+
+// --lds-service: which lanes of a wavefront the LDS serves together, and over how many bytes its banks repeat,
+// for each kind of access.  One dispatch of imex_probe_lds_pair per question, a single wavefront with two active
+// lanes that access different addresses a given distance apart, 64 times: the dispatch counts bank-conflict
+// cycles (rocprofv3 --pmc SQ_LDS_BANK_CONFLICT) exactly when the two lanes are served in the same pass AND the
+// distance is a multiple of the bank period.  Per kind: lane 0 against every other lane, 1024 bytes apart
+// (a multiple of every candidate period), then lanes 0 and 1 at 16 .. 1024 bytes.  Prints the question of every
+// dispatch in launch order, which is the order of the counter file's Dispatch_Id.
+int runLdsServiceProbe() {
+  static const char *kinds[6] = {"ds_read_b128", "ds_write_b128", "ds_read_b64", "ds_write_b64", "ds_read_b32", "ds_write_b32"};
+  const std::vector<char> &image = probeImage();
+  if (image.empty()) {
+    fprintf(stderr, "--lds-service: cannot read %s/imex_probe.hsaco\n", programDir().c_str());
+    return 1;
+  }
+  void *stream = gpuCreateStream(nullptr, nullptr);
+  void *module = gpuModuleLoad(stream, image.data(), image.size());
+  void *kernel = gpuKernelGet(stream, module, "imex_probe_lds_pair");
+  void *out = gpuMemAlloc(stream, 256, 64, /*isShared=*/0);
+  ImexEventDesc noDeps[1] = {{nullptr}};
+  int n = 0;
+  auto ask = [&](int64_t kind, int64_t lane, int64_t bytesApart) {
+    ImexParamDesc ps[5] = {{&out, sizeof(void *)}, {&kind, 8}, {&lane, 8}, {&bytesApart, 8}, {nullptr, 0}};
+    gpuLaunchKernel(stream, kernel, 1, 1, 1, 64, 1, 1, 0, ps, noDeps);
+    gpuWait(stream);
+    printf("dispatch %d: %s lanes 0 and %d, %d bytes apart\n", ++n, kinds[kind], static_cast<int>(lane),
+           static_cast<int>(bytesApart));
+  };
+  for (int kind = 0; kind < 6; ++kind) {
+    for (int lane = 1; lane < 64; ++lane)
+      ask(kind, lane, 1024);
+    for (int bytes = 16; bytes <= 1024; bytes *= 2)
+      ask(kind, 1, bytes);
+  }
+  gpuMemFree(stream, out);
+  gpuStreamDestroy(stream);
+  return 0;
+}
+
 int runWorkload(const Workload &w, const Options &opt) {
   void *stream = gpuCreateStream(nullptr, nullptr);
   std::vector<void *> dev;
@@ -341,21 +396,13 @@ int runWorkload(const Workload &w, const Options &opt) {
   size_t grid[3] = {1, 1, 1}, block[3] = {static_cast<size_t>(w.probeBlock), 1, 1}, smem = 0;
   size_t blobSize = 0;
   const void *blob = nullptr;
-  static std::vector<char> probeBlob; // kept for the life of the process: the runtime caches modules by address
   if (w.probe) {
     grid[0] = w.probeGrid ? static_cast<size_t>(w.probeGrid)
                           : static_cast<size_t>((w.dims[0] + w.probeBlock - 1) / w.probeBlock);
+    const std::vector<char> &probeBlob = probeImage();
     if (probeBlob.empty()) {
-      const std::string path = programDir() + "/imex_probe.hsaco";
-      FILE *f = fopen(path.c_str(), "rb");
-      if (!f) {
-        fprintf(stderr, "%s: cannot read %s\n", w.name, path.c_str());
-        return 1;
-      }
-      char buf[65536];
-      for (size_t n; (n = fread(buf, 1, sizeof buf, f)) > 0;)
-        probeBlob.insert(probeBlob.end(), buf, buf + n);
-      fclose(f);
+      fprintf(stderr, "%s: cannot read %s/imex_probe.hsaco\n", w.name, programDir().c_str());
+      return 1;
     }
     blob = probeBlob.data();
     blobSize = probeBlob.size();
@@ -504,6 +551,8 @@ int main(int argc, char **argv) {
       for (const Workload &w : all)
         printf("%s  (%s)\n", w.name, w.kernel);
       return 0;
+    } else if (a == "--lds-service") {
+      return runLdsServiceProbe();
     } else if (a == "-l" || a == "-s") {
       // backend selectors of bench_imex (Level Zero / SYCL); HIP is the only runtime here
     } else if (a == "-c") {
@@ -541,7 +590,7 @@ int main(int argc, char **argv) {
   }
   if (names.empty() || opt.runs < 1 || opt.rotate < 1 || opt.rotate > 64) {
     fprintf(stderr, "usage: imex-hip-bench [-l] [--runs N] [--warmups W] [--flush] [--zeros] [--rotate S] [--grid G] [--launch-only N] [--report FILE] <workload>|all ...\n"
-                    "       imex-hip-bench --list\n");
+                    "       imex-hip-bench --list\n       imex-hip-bench --lds-service\n");
     return 2;
   }
   for (const std::string &n : names) {

@@ -265,3 +265,36 @@ IMEX_TILE_TRAFFIC(512, 256, 512)
 IMEX_TILE_TRAFFIC(256, 512, 512)
 IMEX_TILE_TRAFFIC(1024, 128, 512)
 IMEX_TILE_TRAFFIC(512, 512, 1024)
+
+// ---- LDS service: which lanes an LDS access serves together, and the bank period ---------------------------
+// imex_probe_lds_pair(out, kind, lane, bytes_apart): one wavefront; lanes 0 and `lane` alone access LDS 64 times,
+// lane 0 at offset 0 and the other at offset bytes_apart, with the access kind 0 .. 5 = 128-bit read, 128-bit
+// write, 64-bit read, 64-bit write, 32-bit read, 32-bit write.  Two lanes that are served in one pass and whose
+// addresses fall into the same bank cost a bank-conflict cycle per access (SQ_LDS_BANK_CONFLICT of the dispatch:
+// 64 or 0); lanes served in different passes never do.  Launch: grid 1, block 64.
+extern "C" __global__ __launch_bounds__(64) void imex_probe_lds_pair(uint32_t *out, int64_t kind, int64_t lane,
+                                                                    int64_t bytes_apart) {
+  using imexhip::u32x2;
+  using imexhip::u32x4;
+  __shared__ __attribute__((aligned(16))) uint32_t words[1024];
+  for (int k = threadIdx.x; k < 1024; k += 64)
+    words[k] = k;
+  __syncthreads();
+  uint32_t acc = 0;
+  const int me = threadIdx.x;
+  if (me == 0 || me == lane) {
+    volatile uint32_t *at = words + (me == 0 ? 0 : (bytes_apart / 4) % 1020);
+    for (int it = 0; it < 64; ++it) {
+      switch (kind) {
+      case 0: acc += (*reinterpret_cast<volatile u32x4 *>(at)).x; break;
+      case 1: *reinterpret_cast<volatile u32x4 *>(at) = u32x4{acc, 1, 2, 3}; break;
+      case 2: acc += (*reinterpret_cast<volatile u32x2 *>(at)).x; break;
+      case 3: *reinterpret_cast<volatile u32x2 *>(at) = u32x2{acc, 1}; break;
+      case 4: acc += *at; break;
+      default: *at = acc; break;
+      }
+    }
+  }
+  if (acc == 0x9e3779b9u) // keeps the reads alive; practically never taken
+    out[me] = acc;
+}
