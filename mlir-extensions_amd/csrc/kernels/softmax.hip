@@ -7,12 +7,15 @@
 //
 // Here: ONE kernel, input read once from HBM and output written once.
 //  * rows of up to 128 lanes x 16 B (1024 16-bit / 512 f32 elements): a
-//    wavefront owns a row (two from 16384 rows on, all loads issued before the
-//    first reduction) and keeps it in registers; max and sum are wavefront-64
-//    butterfly reductions.  Eight wavefronts per SIMD (a 64-register budget) keep
-//    enough loads in flight to cover HBM latency.  With two rows per wavefront the
-//    benchmark shape fills every wavefront slot of the chip exactly once: 5 %
-//    faster on tensors that sit in the caches, the same when they stream from HBM.
+//    wavefront owns a row and keeps it in registers; max and sum are wavefront-64
+//    reductions on the VALU's cross-lane paths (DPP), no LDS.
+//    f16: a wavefront walks rows w, w + W, ... with the next row's loads in
+//    flight while it computes the current one, and the arithmetic is written for
+//    the instruction count (packed f16 maximum, mixed-precision FMAs straight
+//    from and into the f16 halves, one reciprocal per row): about 6 vector
+//    instructions per element where the generic form below needs 14.
+//    f32 / bf16: the generic form, a wavefront owns one row (two from 16384 rows
+//    on, all loads issued before the first reduction), eight wavefronts per SIMD.
 //  * rows of up to 4096 elements: a workgroup owns a row and stages it in LDS
 //    as f32 (read once, three passes over LDS).
 //  * longer rows: workgroup per row, the streaming form -- a running (max, sum)
@@ -24,7 +27,8 @@
 // Arguments: (in, out, rows: i64, cols: i64).
 // Launch: block (256,1,1); any grid >= 1 is correct (workgroups stride over the
 // rows); the catalogue sizes it to one pass: ceil(rows/4) for register-resident
-// rows (ceil(rows/8) from 16384 rows on), else min(rows, 65535 * 16).
+// rows (ceil(rows/8) from 16384 rows on; f16: min(ceil(rows/4), 2048) -- one
+// wavefront per wavefront slot of the chip), else min(rows, 65535 * 16).
 
 #include "device_common.h"
 

@@ -15,7 +15,9 @@
 //  * 16-bit: R x 128 tile (or two of them side by side, loaded together), the
 //    same scheme on 8 x 8 blocks: a lane's eight row loads are repacked with
 //    v_perm_b32 into eight 128-bit groups of the transposed image, one per
-//    column; 128-bit LDS accesses on both sides, XOR-swizzled by group.
+//    column; 128-bit LDS accesses on both sides, XOR-swizzled by group.  Problems
+//    made of whole 256 x 256 tiles send a tile through LDS a quarter (64 columns)
+//    at a time, while the later quarters are still arriving from memory.
 //  * Tile size: the WRITE side of a transpose is the scattered one, and its row
 //    segments are R elements long.  Measured streaming from HBM, 512-byte write
 //    segments reach 74-78% of peak where 256-byte ones stop at 67-70%, so large
@@ -70,9 +72,10 @@ __device__ __forceinline__ void lds_barrier() {
 // one 128-bit load per row with whole 512-byte row segments per wavefront; the 4 x 4 block is then
 // transposed by picking components -- no data moves between lanes -- and goes to LDS as four 128-bit
 // writes, T[4 v + k][group b].  Output rows leave LDS as 128-bit reads of consecutive groups.  Group g
-// of row c is kept at position g ^ ((c / 4) % 16): the sixteen lanes an LDS access serves together then
-// touch sixteen different 16-byte bank groups on the write side (consecutive v) and on the read side
-// (consecutive g) alike.
+// of row c is kept at position g ^ ((c / 4) % 16): the lanes an LDS access serves together (eight consecutive
+// lanes over 128 bytes of banks for a 128-bit write, sixteen lanes over 256 bytes for a 128-bit read) then
+// touch different 16-byte bank groups on the write side (consecutive v) and on the read side (consecutive
+// g) alike.
 template <int R, int C> struct Tile32 {
   static constexpr int VR = C / 4, BP = kThreads / VR, LP = R / 4 / BP; // load: vectors per row, row blocks per pass, passes
   static constexpr int G = R / 4;                                      // 16-byte groups per LDS row
