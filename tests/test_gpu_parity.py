@@ -208,6 +208,19 @@ def test_softmax_long_rows_streaming_form(host, orc, stream, rows, cols):
     assert close_16(orc, host.softmax(stream, xh, "f16"), orc.softmax_16(xh, "f16"), "f16")
 
 
+@pytest.mark.parametrize("cols,path", [(1024, "registers"), (2000, "lds"), (5000, "streamed")])
+def test_softmax_reciprocal_deviation_is_one_rounding(host, orc, stream, cols, path):
+    """The kernel multiplies by one reciprocal per row where the reference divides per element.  What that may
+    cost, pinned on each of the kernel's three paths: an f16 output is the oracle's divided result or its
+    neighbour (one unit in the last place), and all but a small fraction are the same bits."""
+    say("softmax reciprocal deviation, %s path, cols=%d" % (path, cols))
+    x = orc.fill_normal(64 * cols, "f16", 4242 + cols, 0.0, 2.0).reshape(64, cols)
+    got, ref = host.softmax(stream, x, "f16"), orc.softmax_16(x, "f16")
+    steps = np.abs(got.astype(np.int32) - ref.astype(np.int32))  # positive f16 bit patterns are ordered like their values
+    assert steps.max() <= 1
+    assert np.mean(steps == 0) > 0.98
+
+
 @pytest.mark.parametrize("dtype,cols", [("f32", 20), ("f32", 512), ("f16", 1024), ("f32", 3000), ("f16", 4096),
                                         ("f32", 5000), ("f16", 70000)])
 def test_softmax_nan_and_infinite_rows(host, orc, stream, dtype, cols):
