@@ -299,8 +299,11 @@ def measure_rotating(host, stream, w, passes):
             else:
                 args.append(a)
         sets.append(stream.prepare(w.kernel, w.dims, args))
-    for step in sets:
-        step()
+    # one untimed walk round the ring; MFMA-bound kernels walk it until ~150 launches have gone by, as in
+    # measure_secondary: coming from the allocations and copies above the part needs that long to settle
+    for _ in range(-(-150 // copies) if w.bound == "mfma" else 1):
+        for step in sets:
+            step()
     stream.wait()
     ev0 = stream.timestamp()
     for _ in range(passes):

@@ -185,6 +185,10 @@ std::vector<Workload> workloads() {
       {"gemm_f16_4096_probe_store_nontemporal", "imex_gemm_probe_store_nontemporal", {},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},
+      {"gemm_mlp_bf16_probe_store_nontemporal", "imex_gemm_probe_mlp_store_nontemporal", {},
+       {{Elem::BF16, {K4, K4}, true, -1.7f, 1.7f}, {Elem::BF16, {K4, 11008}, true, -0.035f, 0.035f},
+        {Elem::F32, {11008}, true, -0.17f, 0.17f}, {Elem::BF16, {K4, 11008}, false, 0, 0}},
+       {K4, 11008, K4}, 0, 2.0 * K4 * 11008 * K4, true, true, 688},
       {"gemm_f16_4096_probe_store_lines", "imex_gemm_probe_store_lines", {},
        {{Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F16, {K4, K4}, true, -1, 1}, {Elem::F32, {K4, K4}, false, 0, 0}},
        {K4, K4, K4}, 0, 2.0 * K4 * K4 * K4, true, true, 256},

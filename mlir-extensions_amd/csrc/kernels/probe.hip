@@ -170,6 +170,32 @@ extern "C" __global__ __launch_bounds__(imexhip_gemm::kThreads) void imex_gemm_p
   imexhip_gemm::gemm_entry<imexhip_gemm::F16, false, false>(A, B, M, N, K, imexhip_gemm::StoreF32Lines{C});
 }
 
+// The MLP epilogue with its 8-byte stores marked non-temporal: does keeping the 90 MB output stream out of the
+// last-level cache leave more of it to the operand panels, which every round of tiles fetches again?
+struct BiasSiluBF16NonTemporal {
+  static constexpr bool kColumnsInRegisters = true;
+  uint16_t *out;
+  const float *bias;
+  __device__ __forceinline__ void operator()(int64_t m, int64_t n, int64_t N, float acc) const {
+    imexhip_gemm::BiasSiluBF16{out, bias}(m, n, N, acc);
+  }
+  __device__ __forceinline__ void vec4(int64_t m, int64_t n, int64_t N, imexhip::f32x4 acc) const {
+    const imexhip::f32x4 b = *reinterpret_cast<const imexhip_gemm::f32x4u *>(bias + n);
+    imexhip::u32x2 o;
+    uint16_t h[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      h[r] = imexhip_gemm::bf16_bits_hw(imexhip_gemm::silu_fast(acc[r] + b[r]));
+    o.x = h[0] | (uint32_t(h[1]) << 16);
+    o.y = h[2] | (uint32_t(h[3]) << 16);
+    __builtin_nontemporal_store(o, reinterpret_cast<imexhip::u32x2 *>(out + m * N + n));
+  }
+};
+extern "C" __global__ __launch_bounds__(imexhip_gemm::kThreads) void imex_gemm_probe_mlp_store_nontemporal(
+    const uint16_t *A, const uint16_t *B, const float *bias, uint16_t *out, int64_t M, int64_t N, int64_t K) {
+  imexhip_gemm::gemm_entry<imexhip_gemm::BF16, false, false>(A, B, M, N, K, BiasSiluBF16NonTemporal{out, bias});
+}
+
 // ---- tile copy: the 16-bit transpose's memory traffic without the transposition -------------------
 // imex_probe_tile_copy_b16(in, out, rows, cols, mode): the matrix is walked in 256 x 256 tiles of 16-bit
 // elements in the transpose's own order (diagonal by diagonal, one 256-lane workgroup per tile, workgroups
