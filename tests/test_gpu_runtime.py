@@ -300,6 +300,18 @@ def test_driver_runs_every_workload():
         assert any(l.startswith(n + ": back-to-back") for l in r.stdout.splitlines()), n
 
 
+def test_driver_lds_service_probe_mode():
+    """`--lds-service` launches one two-lane LDS probe per question (6 access kinds x (63 lane pairs + 7
+    distances)) and names each dispatch in launch order, which is what a bank-conflict counter run is decoded by."""
+    exe = os.path.join(REPO, "mlir-extensions_amd", "lib", "imex-hip-bench")
+    r = subprocess.run([exe, "--lds-service"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.startswith("dispatch ")]
+    assert len(lines) == 6 * 70
+    assert lines[0] == "dispatch 1: ds_read_b128 lanes 0 and 1, 1024 bytes apart"
+    assert lines[-1] == "dispatch 420: ds_write_b32 lanes 0 and 1, 1024 bytes apart"
+
+
 def test_adopted_stream_and_graph_replay(host, orc):
     """A queue built on a caller's hipStream_t (the `context` argument of gpuCreateStream) launches
     on that stream, so a launch-bound sequence can be captured into a HIP graph and replayed:
