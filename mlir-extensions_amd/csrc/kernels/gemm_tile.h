@@ -18,11 +18,15 @@
 //   registers).  16x16x32 rather than 32x32x16: the two read the same LDS bytes per
 //   FLOP, but on random operands the part sustains about 9 % more with the former
 //   (the shader clock under MFMA load follows the operand values);
-//   K advances 32 at a time through a ring of four 32 KiB LDS stages: A and B
-//   tiles go from global memory STRAIGHT into LDS (buffer_load ... lds, 16 bytes
-//   per lane, no register staging) three steps ahead of the step that multiplies
-//   them; a step waits (vmcnt) only for the oldest tile in flight, then meets the
-//   other wavefronts at the step's single barrier;
+//   K advances 32 at a time; each operand has a ring of four 16 KiB LDS stages,
+//   except that A [M,K] with K % 64 == 0 is copied as slabs of 64 k (128-byte rows:
+//   one L2 request per cache line where 32-k slabs make 64-byte requests) into a
+//   ring of three 32 KiB stages, half a slab with each of the two steps it covers
+//   (160 KiB of LDS in all).  A and B tiles go from global memory STRAIGHT into
+//   LDS (buffer_load ... lds, 16 bytes per lane, no register staging) three steps
+//   ahead of the step that multiplies them; a step waits (vmcnt) only for the
+//   oldest tile in flight, then meets the other wavefronts at the step's single
+//   barrier;
 //   the LDS images are swizzled -- A [256 rows][32 k] by 16-byte group, B
 //   [32 k][256 n] by 32-byte pair -- and because a direct copy fixes each lane's
 //   LDS position, the swizzle is applied to the lane's GLOBAL address instead;
