@@ -350,6 +350,30 @@ def measure_split_k(stream, host):
     return out
 
 
+def measure_tile_rounds(stream):
+    """imex_gemm_bf16_bias_silu_bf16 with M = K = 4096 at N = 2048 .. 16384: half a round, whole rounds and the MLP
+    shape's 2.69 rounds of 256 tiles on the 256 CUs, random operands (numpy generator, seed 5), same buffers back to
+    back: what the last, partial round of tiles costs against whole ones."""
+    rng = np.random.default_rng(5)
+
+    def bf16(x):
+        return (x.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    M = K = 4096
+    a = stream.to_device(bf16(rng.standard_normal((M, K), np.float32)))
+    out = {}
+    for N in (2048, 4096, 8192, 11008, 12288, 16384):
+        b = stream.to_device(bf16(rng.standard_normal((K, N), np.float32) * 0.02))
+        bias = stream.to_device((rng.standard_normal(N) * 0.1).astype(np.float32))
+        o = stream.alloc(M * N * 2)
+        ms = stream.profile("imex_gemm_bf16_bias_silu_bf16", [M, N, K], [a, b, bias, o, M, N, K],
+                            warmups=200, rounds=300, mode=1)[0] / 300
+        out["N=%d" % N] = {"tiles": (M // 256) * -(-N // 256), "ms": round(ms, 5)}
+        for ptr in (b, bias, o):
+            stream.free(ptr)
+    stream.free(a)
+    return out
+
+
 def measure_reference_suite(stream):
     """Every shape and dtype the reference's benchmark suite instantiates (README.md:330-335, benchmarks/*/
     *.shapes.in, *.dtypes.in) plus the two fused chains at their size (512x1024): microseconds per launch over 200
@@ -717,6 +741,8 @@ def main():
         log("reference benchmark suite: %d shapes timed" % len(result["reference_suite_us_per_launch"]))
         result["gemm_bias_silu_split_k_ms_per_launch_MxNxK"] = measure_split_k(stream, host)
         log("split-K operator entry against the plain kernel: %s" % result["gemm_bias_silu_split_k_ms_per_launch_MxNxK"])
+        result["gemm_bias_silu_ms_by_rounds_of_tiles"] = measure_tile_rounds(stream)
+        log("MLP kernel by rounds of tiles: %s" % result["gemm_bias_silu_ms_by_rounds_of_tiles"])
 
     for w in workloads:
         for p in w.buffers:
