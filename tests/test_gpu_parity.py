@@ -502,6 +502,22 @@ def test_loop_fusion_logf_sweep(host, orc, stream):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+def test_empty_inputs_every_operator(host, stream):
+    """Tensors with a zero extent: nothing is launched (a grid of zero workgroups is not a launch), results have
+    the right shape, a row sum over no columns is the initial value and a product over K = 0 is all zeros."""
+    f = np.float32
+    assert host.relu(stream, np.zeros((0,), f)).shape == (0,)
+    assert host.silu(stream, np.zeros((0,), f)).shape == (0,)
+    assert host.softmax(stream, np.zeros((0, 16), f), "f32").shape == (0, 16)
+    assert host.softmax(stream, np.zeros((4, 0), f), "f32").shape == (4, 0)
+    assert host.rowsum(stream, np.zeros((0, 16), f)).shape == (0,)
+    assert np.array_equal(host.rowsum(stream, np.zeros((5, 0), f)), np.zeros(5, f))
+    assert host.transpose2d(stream, np.zeros((0, 7), f)).shape == (7, 0)
+    assert host.transpose2d(stream, np.zeros((7, 0), f)).shape == (0, 7)
+    assert host.gemm(stream, np.zeros((0, 8), np.uint16), np.zeros((8, 16), np.uint16)).shape == (0, 16)
+    assert np.array_equal(host.gemm(stream, np.zeros((4, 0), np.uint16), np.zeros((0, 16), np.uint16)), np.zeros((4, 16), f))
+
+
 def test_fused_chains_empty_and_single(host, orc, stream):
     empty = np.zeros((0,), np.float32)
     assert host.loop_fusion(stream, empty, empty).shape == (0,)
