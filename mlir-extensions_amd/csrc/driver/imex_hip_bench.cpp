@@ -82,6 +82,15 @@ std::vector<Workload> workloads() {
       {"silu_f32_512x640x20x15", "imex_silu_f32", {98304000},
        {{Elem::F32, {98304000}, true, -8, 8}, {Elem::F32, {98304000}, 0, 0, 0}}, {98304000}, 0,
        2.0 * 98304000 * 4, false},
+      {"silu_f16_512x640x20x15", "imex_silu_f16", {98304000},
+       {{Elem::F16, {98304000}, true, -8, 8}, {Elem::F16, {98304000}, 0, 0, 0}}, {98304000}, 0,
+       2.0 * 98304000 * 2, false},
+      {"silu_bf16_512x640x20x15", "imex_silu_bf16", {98304000},
+       {{Elem::BF16, {98304000}, true, -8, 8}, {Elem::BF16, {98304000}, 0, 0, 0}}, {98304000}, 0,
+       2.0 * 98304000 * 2, false},
+      {"relu_f16_512x640x20x15", "imex_relu_f16", {98304000},
+       {{Elem::F16, {98304000}, true, -8, 8}, {Elem::F16, {98304000}, 0, 0, 0}}, {98304000}, 0,
+       2.0 * 98304000 * 2, false},
       {"softmax_f16_16384x1024", "imex_softmax_f16", {16384, 1024},
        {{Elem::F16, {16384, 1024}, true, -4, 4}, {Elem::F16, {16384, 1024}, 0, 0, 0}}, {16384, 1024}, 0,
        2.0 * 16384 * 1024 * 2, false},

@@ -256,24 +256,53 @@ struct ExpF32 {
 // 16-bit SiLU: widen to f32, the same five f32 operations, one rounding back to the 16-bit type
 // (the policy the reference applies to 16-bit element types on the GPU,
 // docs/Transforms/BF16ToGpu.md:17-26; benchmarks/silu/silu.dtypes.in lists f16).
+//
+// A 16-bit type has 65536 inputs, so what the f32 chain must deliver is the right 16-bit result for each
+// of them, not a correctly rounded f32 value in between -- and that can be checked for every input.  The
+// vector path therefore evaluates x * rcp(1 + exp2(-x * log2(e))) with the hardware's exponential and
+// reciprocal estimates (an ulp or two of f32 each, fixed functions of their input on this part):
+//   f16:  the same bits as the libm-exact chain for every one of the 65536 input patterns, NaN and
+//         infinities included, so there is no other case;
+//   bf16: with one Newton step on the reciprocal the same bits for every |x| < 64; beyond that
+//         (exp(-x) near the f32 overflow threshold gives denormal results) the exact chain runs, chosen
+//         once per wavefront and vector like the f32 kernel's general form.
+// A GPU test compares every input pattern of both types with the CPU restatement, so a part or a compiler
+// whose estimates differ cannot go unnoticed.  The exact chain (twelve f64 operations per element) is about
+// 45 vector operations per element where four bytes of traffic leave time for about 24; this form is 8
+// ordinary and 2 quarter-rate ones, and the kernel is memory-bound like ReLU.
 template <io::Dt D> struct Silu16 {
   using E = io::Elem<D>;
   SiluF32 f32;
+  static __device__ __forceinline__ float estimate(float x) {
+    constexpr float kMinusLog2e = -1.44269504088896340736f;
+    const float e = __builtin_amdgcn_exp2f(x * kMinusLog2e);
+    const float d = 1.0f + e;
+    float r = __builtin_amdgcn_rcpf(d);
+    if constexpr (D == io::Dt::BF16)
+      r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+    return x * r;
+  }
   __device__ __forceinline__ u32x4 vec(u32x4 v) const {
     float f[E::kPerVec];
     E::unpack(v, f);
-    bool all = true;
-#pragma unroll
-    for (int i = 0; i < E::kPerVec; ++i)
-      all = all && SiluF32::moderate(f[i]);
-    if (__builtin_amdgcn_ballot_w64(!all) == 0) {
+    if constexpr (D == io::Dt::F16) {
 #pragma unroll
       for (int i = 0; i < E::kPerVec; ++i)
-        f[i] = f32.one_moderate(f[i]);
+        f[i] = estimate(f[i]);
     } else {
+      bool all = true;
 #pragma unroll
       for (int i = 0; i < E::kPerVec; ++i)
-        f[i] = f32.one(f[i]);
+        all = all && SiluF32::moderate(f[i]);
+      if (__builtin_amdgcn_ballot_w64(!all) == 0) {
+#pragma unroll
+        for (int i = 0; i < E::kPerVec; ++i)
+          f[i] = estimate(f[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < E::kPerVec; ++i)
+          f[i] = f32.one(f[i]);
+      }
     }
     return E::pack(f);
   }
